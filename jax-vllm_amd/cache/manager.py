@@ -173,6 +173,12 @@ class CacheManager:
     def slot(self, request_id) -> int:
         return self.requests[request_id].slot
 
+    def last_token(self, request_id) -> int:
+        """The last token whose keys and values the request holds (the one before its next token), -1 before
+        its first: part of a sequence's state for models whose embedding looks at a token's predecessor."""
+        tokens = self.requests[request_id].tokens
+        return tokens[-1] if tokens else -1
+
     def commit(self, request_id, token_ids: Sequence[int]) -> None:
         """The step has stored keys and values of these tokens: advance the context, hash the
         pages that became full, give back window pages that no later token will read."""

@@ -1,6 +1,8 @@
-// Attention input for heads whose key and value sizes differ, or whose q/k norm spans the whole
-// projection: from a token's row [q: nq * dk | k: nkv * dk | v: nkv * dv] (plus an optional bias)
-//   q, k  <- RMS norm over ALL of q's (k's) columns at once, times a weight of that size (optional)
+// Attention input for heads whose key and value sizes differ, whose q/k norm spans the whole
+// projection, or whose rows hold more than q, k and v: from a token's row that begins with
+// [q: nq * dk | k: nkv * dk | v: nkv * dv] (plus an optional bias)
+//   q, k  <- RMS norm over ALL of q's (k's) columns at once, times a weight of that size (optional), or
+//            (per_head) over every head on its own, times a weight of dk elements shared by the heads
 //   q, k  <- the first rot_dims elements of every head turned by the token's angles
 //   v     <- v * v_scale
 // and stored in the layout the paged attention kernels read, every head padded with zeros to one size
@@ -17,8 +19,8 @@ attn_prepare_wide_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long 
                          const float* __restrict__ k_w, float eps, const float* __restrict__ cos_sin,
                          int rot_dims, const int* __restrict__ slot_mapping, T* __restrict__ k_pages,
                          T* __restrict__ v_pages, int page_size, int nq, int nkv, int dk, int dv, int dp,
-                         float v_scale) {
-  extern __shared__ float row[];          // q | k, after bias
+                         float v_scale, int per_head) {
+  extern __shared__ float row[];          // q | k, after bias; then (per_head) one inverse root per head
   __shared__ float red[32];
   const long long t = blockIdx.x;
   const int qn = nq * dk, kn = nkv * dk, vn = nkv * dv;
@@ -30,7 +32,19 @@ attn_prepare_wide_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long 
     if (c < qn) sq = fmaf(a, a, sq); else sk = fmaf(a, a, sk);
   }
   float inv_q = 1.f, inv_k = 1.f;
-  if (q_w) {
+  float* inv_head = row + qn + kn;
+  if (q_w && per_head) {
+    __syncthreads();
+    // a wave a head in turns; the sum over a head's elements in a fixed order
+    const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE, nw = blockDim.x / JV_WAVE;
+    for (int hd = wid; hd < nq + nkv; hd += nw) {
+      float s = 0.f;
+      for (int i = lane; i < dk; i += JV_WAVE) s = fmaf(row[hd * dk + i], row[hd * dk + i], s);
+      s = wave_sum(s);
+      if (lane == 0) inv_head[hd] = rsqrtf(s / (float)dk + eps);
+    }
+    __syncthreads();
+  } else if (q_w) {
     sq = block_sum(sq, red);
     sk = block_sum(sk, red);
     inv_q = rsqrtf(sq / (float)qn + eps);
@@ -50,14 +64,15 @@ attn_prepare_wide_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long 
     float val = 0.f;
     if (i < dk) {
       const int c = is_q ? hd * dk + i : qn + (hd - nq) * dk + i;
-      const float inv = is_q ? inv_q : inv_k;
+      const float inv = (q_w && per_head) ? inv_head[hd] : (is_q ? inv_q : inv_k);
       const float* wn = is_q ? q_w : k_w;
-      const int wc = is_q ? c : c - qn;
+      const int wc = per_head ? i : (is_q ? c : c - qn);
       val = row[c] * inv * (wn ? wn[wc] : 1.f);
       if (i < rot_dims) {
         const int j = i < half ? i : i - half;
         const int co = i < half ? c + half : c - half;
-        const float other = row[co] * inv * (wn ? wn[is_q ? co : co - qn] : 1.f);
+        const int wo = per_head ? (i < half ? i + half : i - half) : (is_q ? co : co - qn);
+        const float other = row[co] * inv * (wn ? wn[wo] : 1.f);
         const float cs = cos_sin[t * rot_dims + j], sn = cos_sin[t * rot_dims + half + j];
         val = i < half ? val * cs - other * sn : val * cs + other * sn;
       }
@@ -82,18 +97,19 @@ attn_prepare_wide_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long 
                                             const float* q_w, const float* k_w, float eps,                      \
                                             const float* cos_sin, int rot_dims, const int* slot_mapping,        \
                                             void* k_pages, void* v_pages, int page_size, int n, int nq,         \
-                                            int nkv, int dk, int dv, int dp, float v_scale, void* stream) {     \
+                                            int nkv, int dk, int dv, int dp, float v_scale, int per_head,       \
+                                            void* stream) {                                                     \
     if (n <= 0) return 0;                                                                                       \
     if (nq <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || dp < dk || dp < dv || rot_dims < 0 || rot_dims > dk ||     \
         rot_dims % 2 || (rot_dims && !cos_sin) || (!q_w) != (!k_w) || (slot_mapping && (!k_pages || !v_pages))) \
       return (int)hipErrorInvalidValue;                                                                         \
-    const size_t shmem = (size_t)(nq + nkv) * dk * sizeof(float);                                               \
+    const size_t shmem = (size_t)(nq + nkv) * (dk + 1) * sizeof(float);                                         \
     if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;                                                    \
     /* few tokens of many wide heads (a decode step): more threads a token */                                  \
     const int threads = (n <= 256 && (nq + nkv) * dp >= 4096) ? 1024 : 256;                                     \
     hipLaunchKernelGGL(attn_prepare_wide_kernel<T>, dim3(n), dim3(threads), shmem, (hipStream_t)stream, (T*)q_out, \
                        (const T*)qkv, ld, bias, q_w, k_w, eps, cos_sin, rot_dims, slot_mapping, (T*)k_pages,    \
-                       (T*)v_pages, page_size, nq, nkv, dk, dv, dp, v_scale);                                   \
+                       (T*)v_pages, page_size, nq, nkv, dk, dv, dp, v_scale, per_head);                         \
     return JV_LAUNCH_CHECK();                                                                                   \
   }
 

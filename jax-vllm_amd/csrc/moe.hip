@@ -2,8 +2,8 @@
 // grouped matrix products of gated experts.  Nothing here returns to the host: a step's routing is
 // known only on the device, so every launch is sized by upper bounds and blocks without work leave.
 //
-//   route:   z = router logits (float) -> the `top` largest per token (lowest index among equals),
-//            weight = sigmoid(z)
+//   route:   z = router logits (float, plus an optional bias per expert) -> the `top` largest per token
+//            (lowest index among equals), weight = sigmoid(z), or the softmax over the chosen logits alone
 //   group:   entry s = token * top + kk  ->  position in a list ordered by expert; tiles of MOE_TM rows
 //            that never straddle two experts
 //   gate/up: z[pos] = act(w g) * (w u),  g = Wg[e] x[token], u = Wu[e] x[token]      (w = the entry's weight
@@ -19,7 +19,10 @@
 
 // The `top` largest of a token's logits, lowest index among equals: the lanes of a wave scan the token's
 // logits (a copy in LDS), the wave agrees on the best, and the lane that scans the chosen expert takes it out.
-__device__ __forceinline__ void moe_pick(float* zt, int experts, int top, int lane, int* ids, float* weights) {
+#define MOE_SCORE_SIGMOID 0          // weight = sigmoid(logit)
+#define MOE_SCORE_SOFTMAX_CHOSEN 1   // weight = exp(logit) / sum of exp over the token's chosen logits
+__device__ __forceinline__ void moe_pick(float* zt, int experts, int top, int lane, int* ids, float* weights,
+                                         int score) {
   for (int kk = 0; kk < top; ++kk) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
@@ -36,23 +39,35 @@ __device__ __forceinline__ void moe_pick(float* zt, int experts, int top, int la
     if (bi == 0x7fffffff) { bi = kk; bv = __builtin_nanf(""); }      // a row of NaN: some expert, the NaN shows in the output
     if (lane == 0) {
       ids[kk] = bi;
-      weights[kk] = 1.f / (1.f + expf(-bv));
+      weights[kk] = score == MOE_SCORE_SOFTMAX_CHOSEN ? bv : 1.f / (1.f + expf(-bv));
     }
     if ((bi & (JV_WAVE - 1)) == lane) zt[bi] = -INFINITY;
+  }
+  if (score == MOE_SCORE_SOFTMAX_CHOSEN && lane == 0) {
+    // the chosen logits came in descending order: the first is their maximum; sums in that order
+    const float m = weights[0];
+    float sum = 0.f;
+    for (int kk = 0; kk < top; ++kk) {
+      const float p = expf(weights[kk] - m);
+      weights[kk] = p;
+      sum += p;
+    }
+    const float inv = 1.f / sum;
+    for (int kk = 0; kk < top; ++kk) weights[kk] *= inv;
   }
 }
 
 // a wave per token, 4 tokens a block
 __global__ void __launch_bounds__(256)
-moe_route_kernel(const float* __restrict__ logits, int n, int experts, int top,
-                 int* __restrict__ ids, float* __restrict__ weights) {
+moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int n, int experts, int top,
+                 int score, int* __restrict__ ids, float* __restrict__ weights) {
   extern __shared__ float zs[];      // [4][experts]
   const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE;
   const long long t = (long long)blockIdx.x * 4 + wid;
   if (t >= n) return;
   float* zt = zs + wid * experts;
-  for (int e = lane; e < experts; e += JV_WAVE) zt[e] = logits[t * experts + e];
-  moe_pick(zt, experts, top, lane, ids + t * top, weights + t * top);
+  for (int e = lane; e < experts; e += JV_WAVE) zt[e] = logits[t * experts + e] + (bias ? bias[e] : 0.f);
+  moe_pick(zt, experts, top, lane, ids + t * top, weights + t * top, score);
 }
 
 // Router and choice in one launch: a block takes up to MOE_RT tokens, their rows in LDS as floats; a wave per
@@ -63,8 +78,9 @@ moe_route_kernel(const float* __restrict__ logits, int n, int experts, int top,
 #define MOE_RT 8
 template <typename T>
 __global__ void __launch_bounds__(1024)
-moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int n, int hidden, int experts, int top, int tb,
-                  int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ logits_out) {
+moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, const float* __restrict__ bias, int n, int hidden,
+                  int experts, int top, int tb, int score, int* __restrict__ ids, float* __restrict__ weights,
+                  float* __restrict__ logits_out) {
   extern __shared__ float rs[];      // x [tb][hidden] | z [tb][experts]
   float* xs = rs;
   float* z = rs + tb * hidden;
@@ -102,7 +118,7 @@ moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int n, int h
 #pragma unroll
     for (int t = 0; t < MOE_RT; ++t) {
       if (t >= nt) continue;
-      const float v = wave_sum(acc[t]);
+      const float v = wave_sum(acc[t]) + (bias ? bias[e] : 0.f);
       if (lane == 0) {
         z[t * experts + e] = v;
         if (logits_out) logits_out[(t0 + t) * experts + e] = v;
@@ -111,7 +127,7 @@ moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int n, int h
   }
   __syncthreads();
   for (int t = wid; t < nt; t += nw)
-    moe_pick(z + t * experts, experts, top, lane, ids + (t0 + t) * top, weights + (t0 + t) * top);
+    moe_pick(z + t * experts, experts, top, lane, ids + (t0 + t) * top, weights + (t0 + t) * top, score);
 }
 
 // One block.  meta: [0] number of tiles; offsets [experts + 1]; tile_expert / tile_row0 [max_tiles];
@@ -281,12 +297,14 @@ moe_down_kernel(float* __restrict__ y, const T* __restrict__ z, const T* __restr
 
 extern "C" int jv_moe_tile_rows() { return MOE_TM; }
 
-extern "C" int jv_moe_route(const float* logits, int n, int experts, int top, int* ids, float* weights, void* stream) {
+extern "C" int jv_moe_route(const float* logits, const float* bias, int n, int experts, int top, int score, int* ids,
+                            float* weights, void* stream) {
   if (n <= 0) return 0;
-  if (experts <= 0 || top <= 0 || top > experts) return (int)hipErrorInvalidValue;
+  if (experts <= 0 || top <= 0 || top > experts || score < 0 || score > MOE_SCORE_SOFTMAX_CHOSEN)
+    return (int)hipErrorInvalidValue;
   if (experts > 3840) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(moe_route_kernel, dim3((n + 3) / 4), dim3(256), 4 * experts * sizeof(float), (hipStream_t)stream,
-                     logits, n, experts, top, ids, weights);
+                     logits, bias, n, experts, top, score, ids, weights);
   return JV_LAUNCH_CHECK();
 }
 
@@ -300,17 +318,19 @@ extern "C" int jv_moe_group(const int* ids, int entries, int experts, int tile_r
 }
 
 #define DEFINE_MOE(SUF, T)                                                                                        \
-  extern "C" int jv_moe_router_##SUF(const void* x, const void* W, int n, int hidden, int experts, int top,       \
-                                     int* ids, float* weights, float* logits_out, void* stream) {                 \
+  extern "C" int jv_moe_router_##SUF(const void* x, const void* W, const float* bias, int n, int hidden,          \
+                                     int experts, int top, int score, int* ids, float* weights,                   \
+                                     float* logits_out, void* stream) {                                           \
     if (n <= 0) return 0;                                                                                         \
-    if (experts <= 0 || top <= 0 || top > experts || hidden <= 0 || (hidden + experts) > 15000)                   \
+    if (experts <= 0 || top <= 0 || top > experts || hidden <= 0 || (hidden + experts) > 15000 || score < 0 ||    \
+        score > MOE_SCORE_SOFTMAX_CHOSEN)                                                                         \
       return (int)hipErrorInvalidValue;                                                                           \
     int tb = 15000 / (hidden + experts);             /* tokens of a block: their rows and logits in 60 KB */      \
     tb = tb > MOE_RT ? MOE_RT : tb;                                                                               \
     while (tb > 1 && (n + tb - 1) / tb < 128) --tb;  /* few tokens: more blocks rather than rows sharing a read */ \
     hipLaunchKernelGGL(moe_router_kernel<T>, dim3((n + tb - 1) / tb), dim3(1024),                                  \
                        (size_t)tb * (hidden + experts) * sizeof(float), (hipStream_t)stream, (const T*)x,         \
-                       (const T*)W, n, hidden, experts, top, tb, ids, weights, logits_out);                       \
+                       (const T*)W, bias, n, hidden, experts, top, tb, score, ids, weights, logits_out);          \
     return JV_LAUNCH_CHECK();                                                                                     \
   }                                                                                                               \
   extern "C" int jv_moe_gate_up_##SUF(void* z, const void* x, const void* Wg, const void* Wu, const int* meta,    \

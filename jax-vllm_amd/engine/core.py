@@ -51,7 +51,7 @@ class _DecodeGraph:
 
     def __init__(self, rb: int, widths: tuple, n_groups: int, device):
         names = [("tokens", rb), ("positions", rb), ("token_req", rb), ("cu", rb + 1), ("ctx", rb), ("slots", rb),
-                 ("rows", rb)]
+                 ("rows", rb), ("prev", rb)]
         names += [(f"slot_mapping{g}", rb) for g in range(n_groups)]
         names += [(f"table{g}", rb * widths[g]) for g in range(n_groups)]
         self.rb, self.widths, self.n_groups = rb, widths, n_groups
@@ -95,6 +95,7 @@ class _DecodeGraph:
             slot_mappings=[self.dev_segment(f"slot_mapping{g}") for g in range(self.n_groups)],
             page_size=page_size, q_lens_host=[1] * rb, context_lens_host=[max_kv_len - 1] * rb,
             slot_ids_host=None, max_q_len=1, max_kv_len=max_kv_len, captured=True,
+            token_ids=self.dev_segment("tokens"), prev_tokens=self.dev_segment("prev"),
         )
 
 
@@ -243,6 +244,8 @@ class EngineCore:
         ctx_lens = [rc.context_len for rc in reqs]
         for name in ("tokens", "positions", "ctx"):
             seg(host, name)[r:] = 0
+        seg(host, "prev")[r:] = -1
+        seg(host, "prev")[:r] = [rc.tokens[-1] if rc.tokens else -1 for rc in reqs]
         seg(host, "slots")[r:] = self._spare_slot
         seg(host, "tokens")[:r] = [int(e.tokens[0]) for e in entries]
         seg(host, "positions")[:r] = ctx_lens
@@ -317,7 +320,7 @@ class EngineCore:
         widths = [max(1, max(len(t) for t in tables[g])) for g in range(n_groups)]
         m = sum(len(e.want) for e in entries)
 
-        sizes = [n, n, n, r + 1, r, r, m] + [n] * n_groups + [r * w for w in widths]
+        sizes = [n, n, n, r + 1, r, r, m] + [n] * n_groups + [r * w for w in widths] + [n]
         offsets = np.concatenate([[0], np.cumsum(sizes)])
         buf = torch.empty(int(offsets[-1]), dtype=torch.int32, pin_memory=True)
         host = buf.numpy()
@@ -326,11 +329,14 @@ class EngineCore:
             return host[offsets[i]:offsets[i + 1]]
 
         tok, pos, treq, cu, ctxl, slot_ids, rows = (seg(i) for i in range(7))
+        prev = seg(7 + 2 * n_groups)     # the token before each token in its request: a portion's first one comes from the cache manager
         cu[0] = 0
         at, row_at = 0, 0
         for i, e in enumerate(entries):
             ql = q_lens[i]
             tok[at:at + ql] = np.asarray(e.tokens, dtype=np.int32)
+            prev[at] = cache.last_token(e.request_id)
+            prev[at + 1:at + ql] = tok[at:at + ql - 1]
             pos[at:at + ql] = np.arange(ctx_lens[i], ctx_lens[i] + ql, dtype=np.int32)
             treq[at:at + ql] = i
             for w in e.want:
@@ -363,6 +369,7 @@ class EngineCore:
             slot_mappings=[dseg(7 + g) for g in range(n_groups)],
             page_size=ps, q_lens_host=q_lens, context_lens_host=ctx_lens, slot_ids_host=slots,
             max_q_len=max(q_lens), max_kv_len=max(c + q for c, q in zip(ctx_lens, q_lens)),
+            token_ids=dseg(0), prev_tokens=dseg(7 + 2 * n_groups),
         )
         ctx.extras["pinned"] = buf  # keeps the staging buffer alive until the step has run
         return dseg(0), ctx, dseg(6)

@@ -232,6 +232,91 @@ def scaled_sum(out: torch.Tensor, y, scale: float) -> None:
               c_longlong(0 if parts is None else parts.stride(0)), c_longlong(out.numel()), c_float(scale), _stream()), "scaled_sum")
 
 
+def embedding_pair(h: torch.Tensor, table: torch.Tensor, pair: torch.Tensor, ids: torch.Tensor, prev: torch.Tensor,
+                   buckets: int, mul_prev: int, mul_cur: int) -> None:
+    """h[t] = float(table[ids[t]]) + float(pair[r]) with r = (prev[t] * mul_prev + ids[t] * mul_cur) mod buckets, or
+    r = buckets (the last row of ``pair``) where prev[t] < 0: a sequence's first token."""
+    _dev(h, table, pair, ids, prev)
+    n, hidden = h.shape
+    _f32(h, "h")
+    _i32(ids, "ids", n)
+    _i32(prev, "prev", n)
+    _need(table.dim() == 2 and table.shape[1] == hidden and table.is_contiguous(), "table width differs from h")
+    _need(pair.shape == (buckets + 1, hidden) and pair.dtype == table.dtype and pair.is_contiguous(),
+          "the pair table must be [buckets + 1, hidden] of the table's type")
+    _need(buckets > 0 and 0 <= mul_prev < 2 ** 31 and 0 <= mul_cur < 2 ** 31, "buckets must be positive, the multipliers below 2^31")
+    fn = getattr(library.core(), f"jv_embedding_pair_{_suffix(table.dtype)}")
+    _check(fn(_ptr(h), _ptr(table), _ptr(pair), _ptr(ids), _ptr(prev), c_int(n), c_int(hidden), c_int(table.shape[0]),
+              c_longlong(buckets), c_longlong(mul_prev), c_longlong(mul_cur), _stream()), "embedding_pair")
+
+
+def add_outputs(h: torch.Tensor, a, b=None, out_dtype=None):
+    """h += a + b in the float residual stream (the sum of the two first, then the stream), where ``a`` and ``b`` are
+    what two sublayers returned: rows of the activation type, a float stack [P, rows, width] of partial results
+    (added in order), a pair (rows or None, stack or None), or None.  With ``out_dtype`` returns the new h in
+    that type."""
+    ra, pa = split_sublayer_output(a) if a is not None else (None, None)
+    rb, pb = split_sublayer_output(b) if b is not None else (None, None)
+    _dev(h, ra, pa, rb, pb)
+    _f32(h, "h")
+    _need(h.is_contiguous(), "h must be contiguous")
+    kinds = {t.dtype for t in (ra, rb) if t is not None}
+    _need(len(kinds) <= 1 and (out_dtype is None or not kinds or kinds == {out_dtype}), "rows and the output must have one type")
+    kind = next(iter(kinds), out_dtype or torch.float32)
+    for t in (ra, rb):
+        _need(t is None or (t.shape == h.shape and t.is_contiguous()), "rows must match h's shape")
+    for t in (pa, pb):
+        _need(t is None or (t.dtype == torch.float32 and t.dim() == 3 and t.shape[1:] == h.shape and t[0].is_contiguous()),
+              "parts must be float32 [P, *h.shape]")
+    out = torch.empty(h.shape, dtype=out_dtype, device=h.device) if out_dtype is not None else None
+    n = h.numel()
+    strides = [t.stride(0) if t is not None else 0 for t in (pa, pb)]
+    vec = h.shape[1] % 4 == 0 and all(s % 4 == 0 for s in strides) and all(
+        t is None or t.data_ptr() % 16 == 0 for t in (h, ra, pa, rb, pb, out))
+    fn = getattr(library.core(), f"jv_add_outputs_{_suffix(kind)}")
+    _check(fn(_ptr(h), _ptr(ra), _ptr(pa), c_int(0 if pa is None else pa.shape[0]), c_longlong(strides[0]),
+              _ptr(rb), _ptr(pb), c_int(0 if pb is None else pb.shape[0]), c_longlong(strides[1]), _ptr(out),
+              c_longlong(n), c_int(1 if vec else 0), _stream()), "add_outputs")
+    return out
+
+
+def token_gate_mul(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, offset: int, activation="gelu_tanh") -> None:
+    """z[t, c] = act(z[t, c]) * table[ids[t], offset + c] in place for contiguous rows z [n, dim]; ``activation`` one
+    of ``PLAIN_ACTIVATIONS``, computed in float."""
+    _dev(z, table, ids)
+    n, dim = z.shape
+    _i32(ids, "ids", n)
+    _need(z.is_contiguous() and table.dim() == 2 and table.is_contiguous() and table.dtype == z.dtype,
+          "z and the table must be contiguous and of one type")
+    _need(0 <= offset and offset + dim <= table.shape[1], "the columns lie outside the table")
+    _need(activation in PLAIN_ACTIVATIONS, f"no kernel for the activation {activation!r}")
+    fn = getattr(library.core(), f"jv_token_gate_mul_{_suffix(z.dtype)}")
+    _check(fn(_ptr(z), _ptr(table), _ptr(ids), c_longlong(n), c_int(dim), c_int(table.shape[1]), c_int(offset),
+              c_int(table.shape[0]), c_int(PLAIN_ACTIVATIONS[activation]), _stream()), "token_gate_mul")
+
+
+def sigmoid_gate_heads(o: torch.Tensor, gate: torch.Tensor, heads: int, dv: int, dp: int) -> None:
+    """o[t, h * dp + i] *= sigmoid(gate[t, h * dv + i]) for i < dv, in place: o [n, heads * dp] contiguous, ``gate`` a
+    [n, heads * dv] view with unit column stride (any row stride) of the same type."""
+    _dev(o)
+    n = o.shape[0]
+    _need(o.is_contiguous() and o.shape == (n, heads * dp) and dp >= dv, "o must be [n, heads * dp]")
+    _need(gate.is_cuda and gate.dtype == o.dtype and gate.shape == (n, heads * dv) and (n == 0 or gate.stride(1) == 1),
+          "gate must be a [n, heads * dv] view with unit column stride")
+    fn = getattr(library.core(), f"jv_sigmoid_gate_heads_{_suffix(o.dtype)}")
+    _check(fn(_ptr(o), _ptr(gate), c_longlong(gate.stride(0)), c_longlong(n), c_int(heads), c_int(dv), c_int(dp), _stream()),
+           "sigmoid_gate_heads")
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap) in place (float32, contiguous)."""
+    _dev(logits)
+    _f32(logits, "logits")
+    _need(logits.is_contiguous() and cap > 0, "contiguous logits and a positive cap")
+    _check(library.core().jv_softcap_f32(_ptr(logits), c_longlong(logits.numel()), c_float(cap), _stream()), "softcap")
+    return logits
+
+
 # --------------------------------------------------------------------------- activation
 GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}      # the kernels' ids of act in y = act(gate) * up
 
@@ -341,24 +426,27 @@ def padded_head_dim(dk: int, dv: int) -> int:
 
 
 def attn_prepare_wide(qkv, bias, q_weight, k_weight, eps: float, cos_sin, rot_dims: int, slot_mapping, k_pages, v_pages,
-                      page_size: int, nq: int, nkv: int, dk: int, dv: int, dp: int, v_scale: float = 1.0) -> torch.Tensor:
-    """Attention input whose key and value sizes differ or whose q/k norm spans the whole projection.  ``qkv`` rows
-    are [q: nq * dk | k: nkv * dk | v: nkv * dv]; ``bias`` (float32, that width) is added first; with
-    ``q_weight`` [nq * dk] and ``k_weight`` [nkv * dk] q and k are RMS-normed over all their columns at once; the
+                      page_size: int, nq: int, nkv: int, dk: int, dv: int, dp: int, v_scale: float = 1.0,
+                      norm_per_head: bool = False) -> torch.Tensor:
+    """Attention input whose key and value sizes differ, whose q/k norm spans the whole projection, or whose rows
+    carry more than q, k and v.  ``qkv`` rows
+    begin with [q: nq * dk | k: nkv * dk | v: nkv * dv] (further columns are left alone); ``bias`` (float32, that width) is added first; with
+    ``q_weight`` [nq * dk] and ``k_weight`` [nkv * dk] q and k are RMS-normed over all their columns at once (with
+    ``norm_per_head``: every head on its own, with weights [dk] shared by the heads); the
     first ``rot_dims`` elements of every q and k head turn by ``cos_sin`` (``rope_table``); v is multiplied by
     ``v_scale``.  Returns q as [n, nq * dp] with every head padded with zeros to ``dp``; keys go to
     [pages, nkv, page_size, dp], values to [pages, nkv, dp, page_size] (their pad is never written)."""
     _dev(qkv, bias, q_weight, k_weight, cos_sin, slot_mapping, k_pages, v_pages)
     n, ld = qkv.shape
     width = (nq + nkv) * dk + nkv * dv
-    _need(ld == width, "qkv must be [tokens, nq * dk + nkv * dk + nkv * dv]")
+    _need(qkv.dim() == 2 and ld >= width and qkv.is_contiguous(), "qkv rows must begin with nq * dk + nkv * dk + nkv * dv columns")
     _need(dp >= max(dk, dv), "the padded head size must hold keys and values")
     if bias is not None:
         _f32(bias, "bias", width)
     _need((q_weight is None) == (k_weight is None), "q and k are normed together or not at all")
     if q_weight is not None:
-        _f32(q_weight, "q_weight", nq * dk)
-        _f32(k_weight, "k_weight", nkv * dk)
+        _f32(q_weight, "q_weight", dk if norm_per_head else nq * dk)
+        _f32(k_weight, "k_weight", dk if norm_per_head else nkv * dk)
     _need(rot_dims % 2 == 0 and 0 <= rot_dims <= dk, "the rotated size must be even and at most the key size")
     if rot_dims:
         _f32(cos_sin, "cos_sin", n * rot_dims)
@@ -370,7 +458,7 @@ def attn_prepare_wide(qkv, bias, q_weight, k_weight, eps: float, cos_sin, rot_di
     _check(fn(_ptr(q), _ptr(qkv), c_longlong(ld), _ptr(bias), _ptr(q_weight), _ptr(k_weight), c_float(eps),
               _ptr(cos_sin if rot_dims else None), c_int(rot_dims), _ptr(slot_mapping if k_pages is not None else None),
               _ptr(k_pages), _ptr(v_pages), c_int(page_size), c_int(n), c_int(nq), c_int(nkv), c_int(dk), c_int(dv),
-              c_int(dp), c_float(v_scale), _stream()), "attn_prepare_wide")
+              c_int(dp), c_float(v_scale), c_int(1 if norm_per_head else 0), _stream()), "attn_prepare_wide")
     return q
 
 
@@ -1375,10 +1463,15 @@ class MoePlan:
         self.tile_rows = tile_rows
 
 
+ROUTER_SCORES = {"sigmoid": 0, "softmax_chosen": 1}      # the kernels' ids of how a chosen logit becomes a weight
+
+
 def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, logits_out=None,
-              tile_rows: "int | None" = None) -> MoePlan:
-    """Chooses for every token the ``top`` experts with the largest router logits (weights sigmoid(logit);
-    the lowest index among equal logits) and orders the n * top entries by expert, all on the device.
+              tile_rows: "int | None" = None, bias=None, score: str = "sigmoid") -> MoePlan:
+    """Chooses for every token the ``top`` experts with the largest router logits (the lowest index among equal
+    logits) and orders the n * top entries by expert, all on the device.  ``bias`` (float32 [experts]) is added
+    to the logits before the choice; ``score``: a chosen expert's weight is "sigmoid" of its logit, or
+    "softmax_chosen": the softmax over the token's chosen logits alone.
     Either float ``logits`` [n, experts] are given, or rows ``x`` [n, hidden] and the router matrix
     ``w_router`` [experts, hidden] of one type: then the logits are made here, in float (``logits_out``,
     float32 [n, experts], receives them if given): in the same launch as the choice (float32, odd sizes), or
@@ -1396,7 +1489,8 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
         elif rows > ROUTER_FUSED_MAX_ROWS:
             logits = gemm_rows_f32out(x, w_router)
         if logits is not None and logits_out is not None:
-            logits_out.copy_(logits)
+            logits_out.copy_(logits if bias is None else logits + bias)
+    _need(score in ROUTER_SCORES, f"no router score {score!r}: there are {sorted(ROUTER_SCORES)}")
     if logits is not None:
         _dev(logits)
         _f32(logits, "logits")
@@ -1412,6 +1506,9 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
             _f32(logits_out, "logits_out", n * experts)
         dev = x.device
     _need(0 < top <= experts, "top must be between 1 and the number of experts")
+    if bias is not None:
+        _dev(bias)
+        _f32(bias, "bias", experts)
     entries = n * top
     tile_rows = tile_rows or moe_tile_rows()
     _need(tile_rows in (64, 128), "tiles have 64 or 128 rows")
@@ -1425,12 +1522,12 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
     weights = torch.empty(entries, dtype=torch.float32, device=dev)
     lib = library.core()
     if logits is not None:
-        _check(lib.jv_moe_route(_ptr(logits), c_int(n), c_int(experts), c_int(top), _ptr(ids), _ptr(weights), _stream()),
-               "moe_route")
+        _check(lib.jv_moe_route(_ptr(logits), _ptr(bias), c_int(n), c_int(experts), c_int(top), c_int(ROUTER_SCORES[score]),
+                                _ptr(ids), _ptr(weights), _stream()), "moe_route")
     else:
         _check(getattr(lib, f"jv_moe_router_{_suffix(x.dtype)}")(
-            _ptr(x), _ptr(w_router), c_int(n), c_int(hidden), c_int(experts), c_int(top), _ptr(ids), _ptr(weights),
-            _ptr(logits_out), _stream()), "moe_router")
+            _ptr(x), _ptr(w_router), _ptr(bias), c_int(n), c_int(hidden), c_int(experts), c_int(top),
+            c_int(ROUTER_SCORES[score]), _ptr(ids), _ptr(weights), _ptr(logits_out), _stream()), "moe_router")
     _check(lib.jv_moe_group(_ptr(ids), c_int(entries), c_int(experts), c_int(tile_rows), _ptr(meta), _ptr(offsets), _ptr(tile_expert),
                             _ptr(tile_row0), _ptr(order), _ptr(rank), _stream()), "moe_group")
     return MoePlan(ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top, tile_rows)

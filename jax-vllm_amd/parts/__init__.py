@@ -1,4 +1,4 @@
-from . import attention, block, embedding, latent_attention, lightning, mlp, moe, norm, recurrent, rotary  # noqa: F401  (register the built-in parts)
+from . import attention, block, embedding, latent_attention, lightning, mlp, moe, norm, recurrent, rotary, token_input  # noqa: F401  (register the built-in parts)
 from .model import DecoderModel, Layer, RunMemoryPlan
 from .spec import (
     PagedCacheSpec,

@@ -24,12 +24,15 @@ class GroupedQueryAttention:
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: Optional[float] = None, position: Optional[PartSpec] = None,
                  window: Optional[int] = None, scale: Optional[float] = None, qkv_bias: bool = False,
-                 o_bias: bool = False, v_head_dim: Optional[int] = None, qk_norm: str = "head", v_scale: float = 1.0):
+                 o_bias: bool = False, v_head_dim: Optional[int] = None, qk_norm: str = "head", v_scale: float = 1.0,
+                 output_gate: bool = False):
         """``v_head_dim``: a value size that differs from the key size; ``qk_norm`` "whole": the q/k norm spans all
         of q's (and all of k's) columns at once, with weights of that size, instead of every head on its own;
-        ``v_scale``: a constant on the values (and so on the mixer's result before its output projection).  Any of
-        the three takes the ``wide`` path: heads cached under one padded size (``K.padded_head_dim``), prepared by
-        ``K.attn_prepare_wide``, read by the same paged attention kernels."""
+        ``v_scale``: a constant on the values (and so on the mixer's result before its output projection);
+        ``output_gate``: the concatenated heads are multiplied by sigmoid(W_g x) before the output projection (W_g is
+        one more block of rows of the fused input projection).  Any of the four takes the ``wide`` path: heads cached
+        under one padded size (``K.padded_head_dim``), prepared by ``K.attn_prepare_wide``, read by the same paged
+        attention kernels."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} q heads are not a multiple of {num_kv_heads} kv heads")
         if qk_norm not in ("head", "whole"):
@@ -38,13 +41,13 @@ class GroupedQueryAttention:
         self.dk = int(head_dim)
         self.dv = int(v_head_dim) if v_head_dim else self.dk
         self.qk_norm, self.v_scale = qk_norm, float(v_scale)
-        self.wide = self.dv != self.dk or (qk_norm == "whole" and qk_norm_eps is not None) or self.v_scale != 1.0
+        self.output_gate = bool(output_gate)
+        self.wide = (self.dv != self.dk or (qk_norm == "whole" and qk_norm_eps is not None) or self.v_scale != 1.0
+                     or self.output_gate)
         # what the paged attention kernels see
         self.d = K.padded_head_dim(self.dk, self.dv) if self.wide else self.dk
         if self.wide:
             self.q_row_stride = self.nq * self.d
-            if qk_norm_eps is not None and qk_norm == "head":
-                raise ValueError("heads of two sizes or scaled values with a q/k norm per head: no kernel prepares that")
         self.qk_norm_eps = qk_norm_eps
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dk)
@@ -80,6 +83,8 @@ class GroupedQueryAttention:
             t["v_proj.bias"] = TensorSpec((self.nkv * self.dv,), role="vector")
         if self.o_bias:
             t["o_proj.bias"] = TensorSpec((self.hidden_size,), role="vector")
+        if self.output_gate:
+            t["gate.weight"] = TensorSpec((self.nq * self.dv, self.hidden_size))
         return t
 
     def cache_spec(self) -> Optional[PagedCacheSpec]:
@@ -90,9 +95,12 @@ class GroupedQueryAttention:
 
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
         self.dtype = dtype
-        self.w_qkv = torch.cat(
-            [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0
-        ).contiguous()
+        # one product for everything that reads the input: q, k, v and, behind them, the gate's rows
+        blocks = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+        if self.output_gate:
+            blocks.append(tensors["gate.weight"])
+        self.w_qkv = torch.cat(blocks, dim=0).contiguous()
+        self.qkv_width = self.nq * self.dk + self.nkv * (self.dk + self.dv)
         self.w_o = tensors["o_proj.weight"]
         if self.wide and self.d != self.dv:
             # the attention's result has heads of the padded size (zeros behind the values): zero columns there
@@ -160,11 +168,14 @@ class GroupedQueryAttention:
         q = K.attn_prepare_wide(
             qkv, self.b_qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos_sin, rotary_dim,
             ctx.slot_mappings[mem.group] if writes else None, mem.pages["k"] if writes else None,
-            mem.pages["v"] if writes else None, ctx.page_size, self.nq, self.nkv, self.dk, self.dv, self.d, self.v_scale)
+            mem.pages["v"] if writes else None, ctx.page_size, self.nq, self.nkv, self.dk, self.dv, self.d, self.v_scale,
+            norm_per_head=self.qk_norm == "head")
         out = torch.empty((qkv.shape[0], self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
         from . import attention_backend
 
         attention_backend.run(self, out, q, ctx, mem)
+        if self.output_gate:
+            K.sigmoid_gate_heads(out, qkv[:, self.qkv_width:], self.nq, self.dv, self.d)
         y = K.linear(out, self.w_o, partial_ok=True)
         if self.b_o is not None:
             K.add_bias(y, self.b_o)

@@ -153,6 +153,55 @@ class OutputNormBlock:
         return K.pending_norm(f, self.norms[1].weight, self.norms[1].eps)
 
 
+class ParallelBlock:
+    """One norm whose output both sublayers read, their outputs joining the stream together, and an optional
+    per-layer token input behind them (``parts/token_input.py``):
+
+        u = norm_1(h);   h = h + (mixer(u) + feed_forward(u));   h = h + norm_t(token_input(h))
+
+    (the feed-forward and the token input are optional).  The sublayers' outputs are added to the float stream by
+    one kernel that also hands the token input the stream in the activation type; the token input's output is
+    handed on as a ``K.PendingNorm`` with its own norm weight (a plain RMS norm), so the next layer's norm (or the
+    final one) does both norms and the residual step in one pass."""
+
+    def __init__(self, norm: PartSpec, has_feed_forward: bool = True, token_input: PartSpec | None = None,
+                 norm_name: str = "norm1", token_input_prefix: str = "side."):
+        self.has_feed_forward = bool(has_feed_forward)
+        self.norm = build_part("norm", norm)
+        self.norm_name, self.token_prefix = norm_name, token_input_prefix
+        self.token_input = build_part("token_input", token_input) if token_input is not None else None
+
+    @property
+    def replayable(self) -> bool:
+        return is_replayable(self.norm) and (self.token_input is None or is_replayable(self.token_input))
+
+    def tensors(self) -> dict:
+        out = {f"{self.norm_name}.{k}": v for k, v in self.norm.tensors().items()}
+        if self.token_input is not None:
+            out.update({self.token_prefix + k: v for k, v in self.token_input.tensors().items()})
+        return out
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        self.dtype = dtype
+        name = self.norm_name + "."
+        self.norm.bind({k[len(name):]: v for k, v in tensors.items() if k.startswith(name)}, dtype)
+        if self.token_input is not None:
+            p = self.token_prefix
+            self.token_input.bind({k[len(p):]: v for k, v in tensors.items() if k.startswith(p)}, dtype)
+
+    def forward(self, h, delta, mixer, feed_forward, ctx, mem):
+        u = self.norm.add_norm(h, delta)
+        a = mixer.forward(u, ctx, mem)
+        f = feed_forward.forward(u, ctx) if self.has_feed_forward else None
+        if self.token_input is None:
+            K.add_outputs(h, a, f)
+            return None
+        x = K.add_outputs(h, a, f, out_dtype=self.dtype)
+        y = self.token_input.forward(x, ctx)
+        return K.pending_norm(y, self.token_input.norm_weight, self.token_input.eps)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "output_norm", OutputNormBlock)
 register_part("block", "sandwich", SandwichBlock)

@@ -35,6 +35,8 @@ class Layer:
 
     def _name(self, sub: str, local: str) -> str:
         below = sub + local
+        if below in self.spec.shared:
+            return self.spec.shared[below]
         return self.spec.prefix + self.spec.rename.get(below, below)
 
     def tensors(self) -> dict:
@@ -126,6 +128,8 @@ class DecoderModel:
     def forward(self, token_ids: torch.Tensor, ctx: StepContext, memories: list, logit_rows: torch.Tensor):
         """Runs the step's tokens through every schedule entry; returns float logits
         [len(logit_rows), vocab] for the token rows named by ``logit_rows`` (int32)."""
+        if ctx.token_ids is None:
+            ctx.token_ids = token_ids
         h = self.embedding.forward(token_ids, ctx)
         delta = None
         for run, mem in zip(self.spec.schedule, memories):

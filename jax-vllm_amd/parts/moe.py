@@ -1,7 +1,8 @@
 """Routed experts: a feed-forward of many small gated feed-forwards, of which each token uses a few
 (no reference counterpart).
 
-    z = W_router x  (float);   s = sigmoid(z);   the ``top`` experts with the largest scores are chosen
+    z = W_router x (+ b)  (float);   the ``top`` experts with the largest z are chosen;
+    s = sigmoid(z), or (``score`` "softmax_chosen") the softmax over the chosen z alone
     out = sum over the chosen e of  expert_e(s_e * x)   [+ shared(x)]
     expert(u) = W_down ( act(W_gate u) * (W_up u) )
 
@@ -24,13 +25,17 @@ from .spec import PartSpec, TensorSpec, build_part, is_replayable, register_part
 class RoutedExperts:
     def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, activation: str = "silu",
                  weight_on_input: bool = True, shared: Optional[PartSpec] = None,
-                 expert_names=("gate", "up", "down")):
+                 expert_names=("gate", "up", "down"), router_bias: bool = False, score: str = "sigmoid"):
         if activation not in K.GATE_ACTIVATIONS:
             raise ValueError(f"the expert kernels have {sorted(K.GATE_ACTIVATIONS)}, not {activation!r}")
         self.hidden_size, self.experts, self.top, self.ff = int(hidden_size), int(num_experts), int(top), int(expert_size)
         if not 0 < self.top <= self.experts:
             raise ValueError(f"top = {self.top} of {self.experts} experts")
+        if score not in K.ROUTER_SCORES:
+            raise ValueError(f"the router kernels have the scores {sorted(K.ROUTER_SCORES)}, not {score!r}")
         self.activation, self.weight_on_input = activation, bool(weight_on_input)
+        self.router_bias, self.score = bool(router_bias), score
+        self.b_router = None
         self.names = tuple(expert_names)
         self.shared = build_part("feed_forward", shared) if shared is not None else None
         if self.shared is not None and hasattr(self.shared, "partial_out"):
@@ -43,6 +48,8 @@ class RoutedExperts:
     def tensors(self) -> dict:
         g, u, d = self.names
         t = {"router.weight": TensorSpec((self.experts, self.hidden_size))}
+        if self.router_bias:
+            t["router.bias"] = TensorSpec((self.experts,), role="vector")
         for e in range(self.experts):
             t[f"experts.{e}.{g}.weight"] = TensorSpec((self.ff, self.hidden_size))
             t[f"experts.{e}.{u}.weight"] = TensorSpec((self.ff, self.hidden_size))
@@ -55,6 +62,8 @@ class RoutedExperts:
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
         g, u, d = self.names
         self.w_router = tensors["router.weight"]
+        if self.router_bias:
+            self.b_router = tensors["router.bias"].contiguous()
         self.w_gate = torch.stack([tensors[f"experts.{e}.{g}.weight"] for e in range(self.experts)]).contiguous()
         self.w_up = torch.stack([tensors[f"experts.{e}.{u}.weight"] for e in range(self.experts)]).contiguous()
         self.w_down = torch.stack([tensors[f"experts.{e}.{d}.weight"] for e in range(self.experts)]).contiguous()
@@ -63,7 +72,7 @@ class RoutedExperts:
 
     def forward(self, x, ctx=None):
         n = x.shape[0]
-        plan = K.moe_route(None, self.top, x=x, w_router=self.w_router,
+        plan = K.moe_route(None, self.top, x=x, w_router=self.w_router, bias=self.b_router, score=self.score,
                            tile_rows=K.moe_tile_rows_for(x.dtype, self.hidden_size, self.ff, n * self.top, self.experts))
         out = torch.empty((self.top, n, self.hidden_size), dtype=torch.float32, device=x.device)
         K.moe_experts(x, plan, self.w_gate, self.w_up, self.w_down, self.activation, out, self.weight_on_input)

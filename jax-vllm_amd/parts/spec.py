@@ -1,7 +1,7 @@
 """The vocabulary that parts, models, cache and engine share.
 
 A *part* is one of: token mixer, feed-forward, norm, position encoding, block
-arrangement, embedding, head.  A part is constructed from its sizes and constants
+arrangement, embedding, head, per-layer token input.  A part is constructed from its sizes and constants
 alone (it never sees a model configuration), declares the tensors it needs under
 local names, and is looked up by ``(category, kind)`` in one registry, so a model
 is a list of ``LayerSpec`` chosen layer by layer plus the order they run in.
@@ -179,6 +179,8 @@ class StepContext:
     extras: dict = field(default_factory=dict)   # per-step results of kernels, shared by parts of one kind
     plans: dict = field(default_factory=dict)    # per-step work lists built on the host and uploaded
     captured: bool = False
+    token_ids: Optional[torch.Tensor] = None     # [N] the step's token ids, for parts inside the layers that look a token up
+    prev_tokens: Optional[torch.Tensor] = None   # [N] the token before each token in its request (-1: the request's first)
 
     @property
     def decode_only(self) -> bool:
@@ -196,7 +198,7 @@ def is_replayable(part) -> bool:
 
 # --------------------------------------------------------------------------- registry of parts
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "token_input")
 _PARTS: dict[tuple, Callable[..., Any]] = {}
 
 
@@ -238,6 +240,9 @@ class LayerSpec:
     feed_forward_prefix: str = ""  # below ``prefix``, e.g. "mlp."
     # local tensor name -> name below ``prefix`` where the checkpoint's differs from the part's
     rename: Mapping[str, str] = field(default_factory=dict)
+    # local tensor name -> full checkpoint name of a tensor that belongs to the model, not to the layer (several
+    # layers may name the same one: it is loaded once and every one of them is handed the same buffer)
+    shared: Mapping[str, str] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
