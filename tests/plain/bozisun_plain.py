@@ -131,6 +131,25 @@ def rotate(x, positions, rot: dict):
 
 
 # --------------------------------------------------------------------------- mixer
+_ONLY_LAST_KEYS = None     # see ``only_last_keys``
+
+
+class only_last_keys:
+    """Within this context every query sees its last ``n`` keys only.  The design has no such limit: a test uses
+    this to show that its rows do hang on keys further back, so that an engine that loses them would be caught."""
+
+    def __init__(self, n: int):
+        self.n = int(n)
+
+    def __enter__(self):
+        global _ONLY_LAST_KEYS
+        self.before, _ONLY_LAST_KEYS = _ONLY_LAST_KEYS, self.n
+
+    def __exit__(self, *exc):
+        global _ONLY_LAST_KEYS
+        _ONLY_LAST_KEYS = self.before
+
+
 def attention(w: dict, p: str, m: dict, u, eps: float):
     """u [n, width], the layer's normed input; positions 0 .. n - 1."""
     n = u.shape[0]
@@ -144,6 +163,8 @@ def attention(w: dict, p: str, m: dict, u, eps: float):
         q, k = rotate(q, range(n), rot), rotate(k, range(n), rot)
     out = torch.zeros(n, H, dv, dtype=u.dtype)
     causal = torch.ones(n, n, dtype=torch.bool).tril()
+    if _ONLY_LAST_KEYS is not None:
+        causal &= torch.ones(n, n, dtype=torch.bool).triu(1 - _ONLY_LAST_KEYS)
     for h in range(H):
         g = h // (H // G)
         s = (q[:, h] @ k[:, g].T) * float(m["scale"])

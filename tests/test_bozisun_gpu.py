@@ -1,0 +1,574 @@
+"""Bozisun on the GPU against its plain implementation (``tests/plain/bozisun_plain.py``): each mechanism alone, whole
+prompts against portions and token-by-token decoding, unequal requests in one batch against each alone, pages and
+slots that are used again, keys at page borders and one far key among hundreds, the first tokens and the token before
+a portion's first one, looped layers with a cache per pass, long decoding through recorded steps, sizes that are no
+multiples of anything, greedy generation through the entry point and its scheduler, and the kernels alone."""
+import numpy as np
+import pytest
+import torch
+
+from tests.bozisun_util import (ALL_SMALL, SMALL_A, SMALL_B, SMALL_C, YARN, attention, check_rows, config, dense, expected,
+                                layer, make_folder, moe, plain_logits, plain_of, rot, tokens_of)
+from tests.plain import bozisun_plain as P
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {s["name"]: make_folder(s, tmp_path_factory.mktemp(f"bz{s['name']}")) for s in ALL_SMALL}
+
+
+def entry(rid, tokens, want=None):
+    from jax_vllm_amd.engine.entries import StepEntry
+
+    return StepEntry(rid, tokens, range(len(tokens)) if want is None else want)
+
+
+def make_core(folder, dtype, page_size, pages=64, seqs=4, graphs=False):
+    from jax_vllm_amd.config import EngineConfig
+    from jax_vllm_amd.engine.core import EngineCore
+    from jax_vllm_amd.weights import load_model
+
+    model, _ = load_model(folder, dtype, "cuda")
+    cfg = EngineConfig(dtype=dtype, block_size=page_size, num_blocks=pages + 1, max_num_seqs=seqs,
+                       max_model_len=pages * page_size, max_num_batched_tokens=4096, enable_prefix_cache=False,
+                       use_hip_graphs=graphs)
+    return EngineCore(model, cfg)
+
+
+def run_cut(core, rid, tokens, cuts):
+    """The request's logits at every position, its tokens fed in portions of the given sizes."""
+    core.start_request(rid)
+    out, at = [], 0
+    for n in cuts:
+        out.append(core.run([entry(rid, tokens[at:at + n])]).cpu().numpy())
+        at += n
+    assert at == len(tokens)
+    core.finish_request(rid)
+    return np.concatenate(out)
+
+
+# ------------------------------------------------------------------ each mechanism alone
+TINY = attention(1, 1, 4, 4)            # the smallest mixer, beside the feed-forward under test
+ALONE = {
+    "attention_groups_and_part_rotation": dict(layers=[layer(attention(4, 2, 12, 20, scale=1.5, rot_=rot(8, 100.0, YARN)))]),
+    "attention_whole_rotation": dict(layers=[layer(attention(3, 3, 10, 6, rot_=rot(10, 1e4)))]),
+    "attention_no_rotation_one_kv_head": dict(layers=[layer(attention(6, 1, 16, 16, scale=0.2))]),
+    "gated_feed_forward": dict(layers=[layer(TINY, dense(72))]),
+    "routed_experts": dict(layers=[layer(TINY, moe(7, 3, 24))]),
+    "routed_experts_one_chosen": dict(layers=[layer(TINY, moe(4, 1, 10))]),
+    "routed_experts_all_chosen": dict(layers=[layer(TINY, moe(3, 3, 16))]),
+    "token_pair_rows": dict(layers=[layer(TINY)], bigram=(23, 7, 11)),
+    "token_input": dict(layers=[layer(TINY), layer(TINY)], side=9),
+    "cap": dict(layers=[layer(TINY)], softcap=2.0),
+    "loop": dict(layers=[layer(attention(2, 1, 8, 8, rot_=rot(4))), layer(attention(2, 2, 8, 12), dense(16))], loop=(0, 1, 3)),
+}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", sorted(ALONE))
+def test_one_mechanism_at_a_time(tmp_path, dtype, which):
+    """A model of one or two layers with one mechanism beside the smallest mixer and nothing else optional: a prompt
+    of 70 tokens whole, and again in portions down to two tokens and single ones."""
+    small = dict(name=which, seed=11, std=0.3, norm_std=0.2, config=config(40, 61, **ALONE[which]))
+    # the cap must bite and the rows per pair must count, or the test shows nothing
+    patch = {"token_pair_rows": {"bigram": lambda t: t * 3.0}}.get(which)
+    folder = make_folder(small, tmp_path, patch)
+    cfg, w = plain_of(folder)
+    toks = tokens_of(cfg, 70, 1)
+    want = expected(cfg, w, toks, dtype)
+    if which == "cap":
+        plain = plain_logits(cfg, w, toks)
+        assert np.abs(plain).max() > 1.9 and 0.1 < (np.abs(plain) > 1.5).mean() < 0.5
+    core = make_core(folder, dtype, 8)
+    check_rows(dtype, run_cut(core, "whole", toks, [70]), want, "whole")
+    check_rows(dtype, run_cut(core, "cut", toks, [2, 3, 1, 17, 2, 31, 1, 1, 2, 10]), want, "portions")
+
+
+# ------------------------------------------------------------------ portions, decoding, first tokens
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("small", ALL_SMALL, ids=[s["name"] for s in ALL_SMALL])
+def test_whole_prompt_portions_and_decoding_agree(folders, dtype, small):
+    cfg, w = plain_of(folders[small["name"]])
+    toks = tokens_of(cfg, 75, 2)
+    want = expected(cfg, w, toks, dtype)
+    core = make_core(folders[small["name"]], dtype, small["page_size"])
+    check_rows(dtype, run_cut(core, "whole", toks, [75]), want, "whole")
+    check_rows(dtype, run_cut(core, "single", toks, [1] * 75), want, "token by token")
+    check_rows(dtype, run_cut(core, "twos", toks, [2] * 37 + [1]), want, "portions of two")
+    check_rows(dtype, run_cut(core, "mixed", toks, [7, 9, 16, 1, 1, 33, 8]), want, "portions of several sizes")
+    check_rows(dtype, run_cut(core, "prompt+decode", toks, [40] + [1] * 35), want, "prompt, then decoding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("small", ALL_SMALL, ids=[s["name"] for s in ALL_SMALL])
+def test_first_tokens_of_a_sequence(folders, dtype, small):
+    """The first token takes the spare row of the pair table and sees one key: prompts of one to five tokens in every cut."""
+    cfg, w = plain_of(folders[small["name"]])
+    toks = [5, 1, 9, 2, 7]
+    want = expected(cfg, w, toks, dtype)
+    core = make_core(folders[small["name"]], dtype, small["page_size"])
+    for rid, cuts in (("one", [1, 1, 1, 1, 1]), ("two", [1, 2, 2]), ("three", [3, 2]), ("whole", [5])):
+        check_rows(dtype, run_cut(core, rid, toks, cuts), want, rid)
+    check_rows(dtype, run_cut(core, "alone", toks[:1], [1]), expected(cfg, w, toks[:1], dtype), "a prompt of one token")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_token_before_a_portion_decides_its_first_row(tmp_path, dtype):
+    """One layer whose mixer is scaled away under a pair table made large, two requests with the same tokens from the
+    second on: the row of the pair (previous, token) carries the logits, so a previous token that is lost at a
+    portion's start, taken from the batch's neighbour or from the slot's last owner moves that row by far more than
+    the tolerance (checked on the plain implementation)."""
+    small = dict(name="pair", seed=13, std=0.3, norm_std=0.1, config=config(32, 50, [layer(TINY)], bigram=(41, 13, 29)))
+    folder = make_folder(small, tmp_path, {"bigram": lambda t: t * 4.0, "l0.mix.o": lambda t: t * 0.05})
+    cfg, w = plain_of(folder)
+    a = tokens_of(cfg, 40, 3)
+    b = [(a[0] + 7) % 50] + a[1:]
+    c = [(t + 3) % 50 for t in a]
+    plain_a, plain_b = plain_logits(cfg, w, a), plain_logits(cfg, w, b)
+    moved = np.abs(plain_a[1] - plain_b[1]).max()
+    assert moved > 0.1 * np.abs(plain_a).max() and np.abs(plain_a[5] - plain_b[5]).max() < 0.05 * moved
+    core = make_core(folder, dtype, 8, seqs=2)
+    for rid, toks in (("a", a), ("b", b)):
+        check_rows(dtype, run_cut(core, rid, toks, [1, 1, 2, 5, 1, 1, 13, 2, 14]), expected(cfg, w, toks, dtype), rid)
+    # side by side in one batch, cut at different places; then a third request in a slot that was used before
+    core.start_request("a")
+    core.start_request("b")
+    got = {"a": [], "b": []}
+    at = {"a": 0, "b": 0}
+    for na, nb in ((1, 3), (2, 1), (1, 1), (7, 2), (1, 9), (28, 24)):
+        out = core.run([entry("a", a[at["a"]:at["a"] + na]), entry("b", b[at["b"]:at["b"] + nb])]).cpu().numpy()
+        got["a"].append(out[:na])
+        got["b"].append(out[na:])
+        at["a"] += na
+        at["b"] += nb
+    core.finish_request("a")
+    core.finish_request("b")
+    check_rows(dtype, np.concatenate(got["a"]), expected(cfg, w, a, dtype), "a beside b")
+    check_rows(dtype, np.concatenate(got["b"]), expected(cfg, w, b, dtype), "b beside a")
+    check_rows(dtype, run_cut(core, "c", c, [1] * 6 + [34]), expected(cfg, w, c, dtype), "a slot used again")
+
+
+# ------------------------------------------------------------------ far keys and page borders
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_one_far_key_among_hundreds_and_page_borders(tmp_path, dtype):
+    """Attention with scores sharp enough that single keys carry a row, as often as not far ones: rows beyond position
+    200 change by much when the plain implementation is kept from seeing keys more than 150 back.  300 tokens over 19
+    pages: whole, in portions that end at, one before and one after page borders, and with the last 40 decoded."""
+    small = dict(name="far", seed=23, std=0.3, norm_std=0.1,
+                 config=config(32, 50, [layer(attention(4, 2, 16, 8, scale=3.0, rot_=rot(8, 1e4, dict(YARN, original=128))))]))
+    folder = make_folder(small, tmp_path)
+    cfg, w = plain_of(folder)
+    toks = tokens_of(cfg, 300, 12)
+    want = expected(cfg, w, toks, dtype)
+    plain = plain_logits(cfg, w, toks)
+    with P.only_last_keys(150):
+        near = plain_logits(cfg, w, toks)
+    assert np.median(np.abs(near[200:] - plain[200:]).max(axis=-1)) > 0.01 * np.abs(plain).max()
+    core = make_core(folder, dtype, 16, pages=20)
+    check_rows(dtype, run_cut(core, "whole", toks, [300]), want, "whole")
+    check_rows(dtype, run_cut(core, "portions", toks, [64, 63, 1, 17, 47, 2, 66] + [1] * 40), want, "portions and decoding")
+    assert core.cache.num_free_pages(0) == 20       # every page came back
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_token_that_occurs_once_is_found_from_everywhere(tmp_path, dtype):
+    """Sharp scores (few keys carry a row) and a token that occurs once, at position 3: the plain implementation
+    shows which later rows hang on that key (their logits move when the token is another one), up to 250 tokens on,
+    over 16 pages; those rows are among the ones compared, in prompts and in decoding."""
+    small = dict(name="one", seed=29, std=0.3, norm_std=0.05,
+                 config=config(32, 50, [layer(attention(2, 1, 16, 16, scale=2.0))]))
+    folder = make_folder(small, tmp_path)
+    cfg, w = plain_of(folder)
+    toks = [t if t != 7 else 8 for t in tokens_of(cfg, 250, 5)]
+    toks[3] = 7
+    other = list(toks)
+    other[3] = 9
+    plain, without = plain_logits(cfg, w, toks), plain_logits(cfg, w, other)
+    want = expected(cfg, w, toks, dtype)
+    # how much the rows at the end hang on position 3 (a sharp softmax picks few keys; this one is among them for
+    # some rows, and those rows are the test)
+    hang = np.abs(plain[100:] - without[100:]).max(axis=-1)
+    assert (hang > 0.02 * np.abs(plain).max()).sum() >= 3
+    core = make_core(folder, dtype, 16, pages=16)
+    check_rows(dtype, run_cut(core, "whole", toks, [250]), want, "whole")
+    check_rows(dtype, run_cut(core, "cut", toks, [3, 1, 12, 16, 15, 2, 31, 100] + [1] * 70), want, "portions and decoding")
+
+
+# ------------------------------------------------------------------ batches, pages and slots used again
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("small", [SMALL_A, SMALL_C], ids=["A", "C"])
+def test_unequal_requests_in_one_batch_with_pages_and_slots_used_again(folders, dtype, small):
+    """Seven requests of 1 to 90 tokens through two slots and a small pool of pages, portions of some beside single
+    tokens of others; each request's logits equal the plain implementation's of it alone."""
+    cfg, w = plain_of(folders[small["name"]])
+    ps = small["page_size"]
+    lengths = [33, 1, 90, 17, 64, 5, 48]
+    reqs = {f"r{i}": tokens_of(cfg, n, 10 + i) for i, n in enumerate(lengths)}
+    want = {r: expected(cfg, w, t, dtype) for r, t in reqs.items()}
+    pages = max(14, 2 * (-(-90 // ps)) + 2)
+    core = make_core(folders[small["name"]], dtype, ps, pages=pages, seqs=2)
+    got = {r: [] for r in reqs}
+    at = {r: 0 for r in reqs}
+    waiting, live = list(reqs), []
+    rng = np.random.default_rng(5)
+    slots_seen = []
+    while waiting or live:
+        while waiting and len(live) < 2:
+            r = waiting.pop(0)
+            core.start_request(r)
+            slots_seen.append(core.cache.slot(r))
+            live.append(r)
+        entries = []
+        for r in live:
+            left = len(reqs[r]) - at[r]
+            n = 1 if (at[r] > 0 and rng.integers(2)) else int(min(left, rng.choice([1, 2, 3, 8, 21])))
+            entries.append(entry(r, reqs[r][at[r]:at[r] + n]))
+            at[r] += n
+        logits = core.run(entries).cpu().numpy()
+        k = 0
+        for e in entries:
+            got[e.request_id].append(logits[k:k + len(e.tokens)])
+            k += len(e.tokens)
+        for r in list(live):
+            if at[r] == len(reqs[r]):
+                core.finish_request(r)
+                live.remove(r)
+        core.cache.check_invariants()
+    assert sorted(set(slots_seen)) == [0, 1] and len(slots_seen) == 7         # slots were used again
+    assert core.cache.num_free_pages(0) == pages
+    if dtype == "float32":
+        for r in reqs:
+            check_rows(dtype, np.concatenate(got[r]), want[r], r)
+    else:       # few rows a request: the shares of rows that rounding moves far are judged over all of them
+        check_rows(dtype, np.concatenate([x for r in reqs for x in got[r]]),
+                   tuple(np.concatenate([want[r][k] for r in reqs]) for k in (0, 1)), "all requests")
+
+
+# ------------------------------------------------------------------ long decoding, recorded steps
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "recorded"])
+def test_long_decoding(folders, dtype, graphs):
+    """260 decoded tokens behind a prompt of 9, over many pages, the looped layers' passes each with its own keys; with
+    recorded steps two requests decode side by side (the shorter one leaves a padded row)."""
+    cfg, w = plain_of(folders["A"])
+    a, b = tokens_of(cfg, 269, 6), tokens_of(cfg, 150, 7)
+    want_a, want_b = expected(cfg, w, a, dtype), expected(cfg, w, b, dtype)
+    core = make_core(folders["A"], dtype, SMALL_A["page_size"], pages=60, graphs=graphs)
+    core.start_request("a")
+    core.start_request("b")
+    got_a = [core.run([entry("a", a[:9])]).cpu().numpy()]
+    got_b = [core.run([entry("b", b[:30])]).cpu().numpy()]
+    for i in range(9, 269):
+        es = [entry("a", a[i:i + 1])]
+        j = 30 + i - 9
+        if j < 150:
+            es.append(entry("b", b[j:j + 1]))
+        out = core.run(es).cpu().numpy()
+        got_a.append(out[:1])
+        if j < 150:
+            got_b.append(out[1:2])
+    check_rows(dtype, np.concatenate(got_a), want_a, "a")
+    check_rows(dtype, np.concatenate(got_b), want_b, "b")
+    if graphs:
+        assert core.graph_replays > 200
+
+
+# ------------------------------------------------------------------ the entry point
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["A", "C"])
+def test_greedy_generation_through_the_entry_point(folders, dtype, which):
+    """Four prompts through ``LLM.generate`` with two slots, a small token budget (prompts are cut) and few pages, decode
+    steps recorded and following each other without the host in between (the token before comes from the cache
+    manager also then): in float32 every token is the plain implementation's argmax; in bfloat16 each token is within a
+    margin of the plain maximum given what came before."""
+    from jax_vllm_amd import LLM, SamplingParams
+
+    small = {"A": SMALL_A, "C": SMALL_C}[which]
+    cfg, w = plain_of(folders[which])
+    prompts = [tokens_of(cfg, n, 30 + n) for n in (3, 41, 18, 70)]
+    llm = LLM(folders[which], dtype=dtype, block_size=small["page_size"], max_num_seqs=2, max_model_len=128,
+              max_num_batched_tokens=24, num_blocks=max(9, 256 // small["page_size"] + 1))
+    assert llm.prewarm() > 0.0
+    got = llm.generate(prompts, SamplingParams(max_new_tokens=12))
+    assert [len(g) for g in got] == [12] * 4
+    assert llm.stats.graph_replays > 0
+    for p, g in zip(prompts, got):
+        seq = list(p)
+        for i, t in enumerate(g):
+            logits = P.forward(w, cfg, seq)[-1]
+            if dtype == "float32":
+                assert int(torch.argmax(logits)) == t, f"token {i}: engine {t}, plain {int(torch.argmax(logits))}"
+            else:
+                assert float(logits.max() - logits[t]) <= 0.06 * float(logits.abs().max()), f"token {i} is far below the maximum"
+            seq.append(t)
+
+
+def test_a_prefix_taken_from_the_cache_keeps_the_token_before(folders):
+    """The design keeps no state beside its pages, so prompts share cached pages; the first computed token behind a
+    cached prefix still finds the token before it."""
+    from jax_vllm_amd import LLM, SamplingParams
+
+    cfg, w = plain_of(folders["A"])
+    ps = SMALL_A["page_size"]
+    shared = tokens_of(cfg, 3 * ps, 77)
+    prompts = [shared + tokens_of(cfg, 5, 78), shared + tokens_of(cfg, 9, 79)]
+    llm = LLM(folders["A"], dtype="float32", block_size=ps, max_num_seqs=1, max_model_len=128, max_num_batched_tokens=64,
+              num_blocks=40, enable_prefix_cache=True)
+    got = llm.generate(prompts, SamplingParams(max_new_tokens=4))
+    assert llm.core.cache.hit_tokens >= 3 * ps
+    for p, g in zip(prompts, got):
+        seq = list(p)
+        for t in g:
+            assert int(torch.argmax(P.forward(w, cfg, seq)[-1])) == t
+            seq.append(t)
+
+
+def test_command_line_runs_the_design(folders, capsys):
+    from jax_vllm_amd.engine.cli import main
+
+    cfg, w = plain_of(folders["B"])
+    prompt = tokens_of(cfg, 12, 40)
+    code = main(["--model-path", str(folders["B"]), "--dtype", "fp32", "--block-size", "16", "--max-model-len", "64",
+                 "--max-prefill-len", "32", "--max-new-tokens", "5", "--no-prewarm", "--prompt-ids",
+                 " ".join(map(str, prompt))])
+    assert code == 0
+    got = [int(t) for t in capsys.readouterr().out.split()]
+    seq = list(prompt)
+    for t in got:
+        assert int(torch.argmax(P.forward(w, cfg, seq)[-1])) == t
+        seq.append(t)
+    assert len(got) == 5
+
+
+class _Both:
+    """(plain logits, plain logits with rounded products) of a request, indexed by position as one."""
+
+    def __init__(self, pair):
+        self.pair = pair
+
+    def __getitem__(self, pos):
+        return self.pair
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_replay_with_four_slots_and_a_pool_for_the_live_requests_only(folders, dtype, tmp_path):
+    """``bin/trace_run`` on a mixed schedule: nine requests of 20 to 150 tokens, at most four live, portions of some
+    beside single tokens of others, some sitting a step out; the pool holds what the live requests hold at the peak, so
+    pages and slots are used again; then one request whole, one with its tail decoded, one in portions down to two."""
+    from tests.replay_util import Trace, compare, mixed, portions, run_trace, tail_one_by_one, whole
+
+    cfg, w = plain_of(folders["A"])
+    rng = np.random.default_rng(17)
+    reqs = {f"q{i}": tokens_of(cfg, n, 50 + i) for i, n in enumerate((150, 20, 77, 64, 33, 129, 48, 90, 65))}
+    trace = Trace()
+    peak = mixed(trace, reqs, rng)
+    whole(trace, "q0#w", reqs["q0"])
+    tail_one_by_one(trace, "q2#t", reqs["q2"], tail=40)
+    portions(trace, "q5#p", reqs["q5"], (2, 31, 3, 17))
+    got = run_trace(folders["A"], dtype, trace, max(peak, 192), tmp_path / "out", block_size=SMALL_A["page_size"])
+    want = {r: expected(cfg, w, t, dtype) for r, t in reqs.items()}
+    rows_got, rows_plain, rows_rounded = [], [], []
+
+    def collect(name, pos, got_row, want_row):
+        rows_got.append(got_row)
+        if dtype == "float32":
+            rows_plain.append(want_row)
+        else:
+            rows_plain.append(want_row[0][pos])
+            rows_rounded.append(want_row[1][pos])
+
+    if dtype == "float32":
+        n = compare(trace, got, want, collect)
+        check_rows(dtype, np.stack(rows_got), np.stack(rows_plain), "trace")
+    else:
+        n = compare(trace, got, {r: _Both(v) for r, v in want.items()}, collect)
+        check_rows(dtype, np.stack(rows_got), (np.stack(rows_plain), np.stack(rows_rounded)), "trace")
+    assert n == sum(len(t) for t in reqs.values()) + 150 + 41 + 129
+
+
+# ------------------------------------------------------------------ other sizes
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_odd_sizes_and_heads_beyond_the_matrix_core_kernels(tmp_path, dtype):
+    """A width that is no multiple of 4, a value size of 260 (above the matrix-core attention kernels: the float kernel
+    runs in bfloat16 too), key sizes of 6 and 10, feed-forwards and experts of odd sizes, a token input of 7 columns,
+    three buckets."""
+    small = dict(name="odd", seed=31, std=0.25, norm_std=0.2, config=config(50, 61, [
+        layer(attention(2, 1, 10, 260, rot_=rot(6)), dense(21)),
+        layer(attention(3, 3, 6, 5, scale=0.8, rot_=rot(2, 10.0, dict(YARN, original=16))), moe(5, 2, 13)),
+        layer(attention(7, 1, 18, 2), None),
+    ], bigram=(3, 1, 1), side=7, loop=(2, 3, 2), softcap=11.0))
+    folder = make_folder(small, tmp_path)
+    cfg, w = plain_of(folder)
+    toks = tokens_of(cfg, 70, 8)
+    want = expected(cfg, w, toks, dtype)
+    core = make_core(folder, dtype, 16)
+    check_rows(dtype, run_cut(core, "whole", toks, [70]), want, "whole")
+    check_rows(dtype, run_cut(core, "cut", toks, [33, 2, 1, 17, 1, 1, 15]), want, "portions")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_wider_layers_and_a_long_prompt(tmp_path, dtype):
+    """Five layers at a width of 256 with heads of 32 to 128 (the sizes at which the matrix-core attention kernels, the
+    matrix-core expert products and the streaming products all run), three of them looped twice, a prompt of 420
+    tokens: whole, in portions that end inside pages, and with a decoded tail."""
+    small = dict(name="wide", seed=41, std=0.08, norm_std=0.1, config=config(256, 500, [
+        layer(attention(6, 3, 32, 64, scale=0.2, rot_=rot(16, 5e4, dict(YARN, original=256, factor=8.0))), dense(320)),
+        layer(attention(4, 4, 64, 32, rot_=rot(64, 1e4)), moe(8, 2, 96)),
+        layer(attention(8, 2, 64, 64, scale=0.15, rot_=rot(32, 1e6)), None),
+        layer(attention(2, 1, 128, 128, rot_=rot(64, 1e4, YARN)), moe(16, 4, 64)),
+        layer(attention(4, 1, 48, 48), dense(192)),
+    ], bigram=(211, 31, 17), side=24, loop=(1, 4, 2), softcap=20.0))
+    folder = make_folder(small, tmp_path)
+    cfg, w = plain_of(folder)
+    toks = tokens_of(cfg, 420, 9)
+    want = expected(cfg, w, toks, dtype)
+    core = make_core(folder, dtype, 16, pages=40)
+    whole, cut = run_cut(core, "whole", toks, [420]), run_cut(core, "cut", toks, [100, 31, 2, 64, 33, 7, 129, 14] + [1] * 40)
+    if dtype == "bfloat16":
+        check_rows(dtype, whole, want, "whole")
+        check_rows(dtype, cut, want, "portions and decoding")
+        return
+    # eight layer runs deep a few positions are badly conditioned (a close choice between experts, a small output in
+    # front of a norm): the plain implementation in float32 is itself off there, so a row may be off by three times
+    # that on top of the usual bound
+    own = np.abs(P.forward(P.read_weights(folder, torch.float32), cfg, toks).numpy().astype(np.float64) - want).max(axis=-1)
+    scale = float(np.abs(want).max())
+    for what, got in (("whole", whole), ("portions and decoding", cut)):
+        err = np.abs(got.astype(np.float64) - want).max(axis=-1)
+        worst = int((err - 3 * own).argmax())
+        assert (err <= 3e-5 * scale + 1e-5 + 3 * own).all(), f"{what}: row {worst} is off by {err[worst]}, plain float32 by {own[worst]}"
+        assert np.median(err) <= 1e-5 * scale, f"{what}: median error {np.median(err)}"
+
+
+# ------------------------------------------------------------------ kernels alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_kernel_embedding_with_pair_rows(dtype):
+    from jax_vllm_amd.ops import kernels as K
+
+    torch.manual_seed(1)
+    vocab, hidden, buckets, a, b = 300, 52, 61, 2147483629, 1000003
+    table = torch.randn(vocab, hidden).to(dtype).cuda()
+    pair = torch.randn(buckets + 1, hidden).to(dtype).cuda()
+    ids = torch.randint(0, vocab, (40,), dtype=torch.int32)
+    prev = torch.randint(0, vocab, (40,), dtype=torch.int32)
+    prev[[0, 7, 39]] = -1
+    h = torch.empty(40, hidden, dtype=torch.float32, device="cuda")
+    K.embedding_pair(h, table, pair, ids.cuda(), prev.cuda(), buckets, a, b)
+    rows = [buckets if p < 0 else (int(p) * a + int(i) * b) % buckets for p, i in zip(prev.tolist(), ids.tolist())]
+    want = table.float().cpu()[ids.long()] + pair.float().cpu()[torch.tensor(rows)]
+    assert torch.equal(h.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("hidden", [48, 50])
+def test_kernel_two_outputs_join_the_stream(dtype, hidden):
+    from jax_vllm_amd.ops import kernels as K
+
+    torch.manual_seed(2)
+    n = 9
+    h0 = torch.randn(n, hidden).cuda()
+    rows = torch.randn(n, hidden).to(dtype).cuda()
+    parts = torch.randn(3, n, hidden).cuda()
+    stack = torch.randn(5, n, hidden).cuda()
+    for a, b in ((rows, parts), (parts, (None, stack)), (rows, None), ((rows, stack), rows)):
+        def total(x):
+            if x is None:
+                return 0.0
+            r, p = x if isinstance(x, tuple) else ((None, x) if x.dim() == 3 else (x, None))
+            return (r.double() if r is not None else 0.0) + (p.double().sum(0) if p is not None else 0.0)
+
+        h = h0.clone()
+        out = K.add_outputs(h, a, b, out_dtype=dtype)
+        want = h0.double() + (total(a) + total(b))
+        assert float((h.double() - want).abs().max()) < 2e-5
+        assert torch.equal(out, h.to(dtype))
+        h2 = h0.clone()
+        assert K.add_outputs(h2, a, b) is None and torch.equal(h2, h)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_kernel_token_gate_heads_gate_and_cap(dtype):
+    from jax_vllm_amd.ops import kernels as K
+
+    torch.manual_seed(3)
+    n, dim, width, off, vocab = 11, 7, 30, 14, 20
+    z = torch.randn(n, dim).to(dtype).cuda()
+    table = torch.randn(vocab, width).to(dtype).cuda()
+    ids = torch.randint(0, vocab, (n,), dtype=torch.int32).cuda()
+    want = P.gelu_tanh(z.double().cpu()) * table.double().cpu()[ids.long().cpu(), off:off + dim]
+    K.token_gate_mul(z, table, ids, off, "gelu_tanh")
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert float((z.double().cpu() - want).abs().max()) < tol
+    # heads padded from 5 to 16 elements, the gate in the tail of a wider row
+    heads, dv, dp = 3, 5, 16
+    o = torch.randn(n, heads * dp).to(dtype).cuda()
+    wide = torch.randn(n, 40 + heads * dv).to(dtype).cuda()
+    want = o.double().cpu().view(n, heads, dp).clone()
+    want[:, :, :dv] *= torch.sigmoid(wide.double().cpu()[:, 40:]).view(n, heads, dv)
+    K.sigmoid_gate_heads(o, wide[:, 40:], heads, dv, dp)
+    assert float((o.double().cpu().view(n, heads, dp) - want).abs().max()) < tol
+    x = (torch.randn(6, 33) * 10).cuda()
+    want = 4.0 * torch.tanh(x.double().cpu() / 4.0)
+    assert float((K.softcap(x, 4.0).double().cpu() - want).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("n", [5, 40, 300])
+def test_kernel_router_with_a_bias_and_the_softmax_over_the_chosen(n):
+    from jax_vllm_amd.ops import kernels as K
+
+    torch.manual_seed(4)
+    hidden, experts, top = 64, 12, 4
+    for dtype in (torch.float32, torch.bfloat16):
+        x = torch.randn(n, hidden).to(dtype)
+        wr = torch.randn(experts, hidden).to(dtype)
+        bias = torch.randn(experts) * 2
+        z = x.double() @ wr.double().T + bias.double()
+        val, idx = torch.topk(z, top, dim=-1)
+        plan = K.moe_route(None, top, x=x.cuda(), w_router=wr.cuda(), bias=bias.cuda(), score="softmax_chosen")
+        torch.cuda.synchronize()
+        ids, wts = plan.ids.cpu().view(n, top).long(), plan.weights.cpu().view(n, top).double()
+        clear = (val[:, :-1] - val[:, 1:]).min(dim=-1).values > 1e-3      # rows whose order no rounding turns
+        clear &= (val[:, -1] - torch.sort(z, dim=-1, descending=True).values[:, top]) > 1e-3
+        assert clear.float().mean() > 0.8
+        assert torch.equal(ids[clear], idx[clear])
+        assert float((wts[clear] - torch.softmax(val[clear], -1)).abs().max()) < 1e-4
+        assert float((wts.sum(-1) - 1).abs().max()) < 1e-5
+        # the choice from given logits with the bias added there is the same choice
+        again = K.moe_route((x.double() @ wr.double().T).float().cuda(), top, bias=bias.cuda(), score="softmax_chosen")
+        assert torch.equal(again.ids.cpu().view(n, top).long()[clear], idx[clear])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_kernel_attention_input_with_a_norm_per_head_and_a_wider_row(dtype):
+    from jax_vllm_amd.ops import kernels as K
+
+    torch.manual_seed(5)
+    n, nq, nkv, dk, dv, dp, rd, ps, extra = 13, 4, 2, 12, 20, 32, 8, 8, 17
+    width = (nq + nkv) * dk + nkv * dv
+    row = torch.randn(n, width + extra).to(dtype)
+    qw, kw = torch.rand(dk) + 0.5, torch.rand(dk) + 0.5
+    pos = torch.arange(n, dtype=torch.int32)
+    inv = 100.0 ** (-torch.arange(0, rd, 2, dtype=torch.float32) / rd)
+    table = K.rope_table(pos.cuda(), inv.cuda())
+    pages = 4
+    kp = torch.zeros(pages + 1, nkv, ps, dp, dtype=dtype, device="cuda")
+    vp = torch.zeros(pages + 1, nkv, dp, ps, dtype=dtype, device="cuda")
+    slots = torch.tensor([(1 + t // ps) * ps + t % ps for t in range(n)], dtype=torch.int32)
+    q = K.attn_prepare_wide(row.cuda(), None, qw.cuda(), kw.cuda(), 1e-5, table, rd, slots.cuda(), kp, vp, ps, nq, nkv, dk, dv,
+                            dp, norm_per_head=True)
+    x = row.double()
+    rot_cfg = {"dims": rd, "base": 100.0}
+    qq = P.rotate(P.rms_norm(x[:, :nq * dk].view(n, nq, dk), qw.double(), 1e-5), range(n), rot_cfg)
+    kk = P.rotate(P.rms_norm(x[:, nq * dk:(nq + nkv) * dk].view(n, nkv, dk), kw.double(), 1e-5), range(n), rot_cfg)
+    vv = x[:, (nq + nkv) * dk:width].view(n, nkv, dv)
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    got = q.double().cpu().view(n, nq, dp)
+    assert float((got[:, :, :dk] - qq).abs().max()) < tol and float(got[:, :, dk:].abs().max()) == 0.0
+    for t in range(n):
+        page, s = 1 + t // ps, t % ps
+        assert float((kp[page, :, s, :dk].double().cpu() - kk[t]).abs().max()) < tol
+        assert float((vp[page, :, :dv, s].double().cpu() - vv[t]).abs().max()) < tol
+    assert float(kp[0].abs().max()) == 0.0 and float(kp[:, :, :, dk:].abs().max()) == 0.0
