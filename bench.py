@@ -4,6 +4,7 @@ prefill tokens/s at 2,048 tokens and decode at batch 1 and 64 beside it.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|14b|32b]
     python bench.py --only design [--design-shape 2k|4k]     # the Lomozen architecture beside the dense model of equal size
     python bench.py --only design --design dumazen           # the Dumazen architecture beside Lomozen and the dense model
+    python bench.py --only design --design bozisun           # the Bozisun architecture beside Lomozen and the dense model
 
 The model has the layer sizes of Qwen3-8B (the headline configuration) with random
 weights drawn on the device; prompts are seeded uniform-random token ids of 1,024 tokens;
@@ -71,6 +72,20 @@ def dumazen_shape(width, layers, heads, ff, vocab=32000, window=1024):
             "layers": [dict(order[i % 4], mlp={"kind": "dense", "ff": ff}) for i in range(layers)]}
 
 
+def bozisun_shape(width, layers, heads, ff, experts, top, expert_ff, loop, vocab=32000):
+    """Attention layers with heads of 128 (a quarter as many kv heads, half of a head rotated with rescaled frequencies, an
+    output gate), a gated feed-forward and routed experts in turns (top * expert_ff = ff), a row per token pair, a
+    per-layer token input of 256 columns, ``loop`` = (start, stop, times) of the layers that run several times."""
+    att = {"type": "attention", "mixer": {
+        "heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+        "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    mlps = ({"kind": "dense", "ff": ff}, {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}})
+    return {"architecture": "Bozisun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "embedding": {"bigram": {"buckets": 100003, "mul_prev": 1000003, "mul_cur": 7919}}, "token_side": {"dim": 256},
+            "loop": dict(zip(("start", "stop", "times"), loop)), "logit_softcap": 30.0,
+            "layers": [dict(att, mlp=mlps[i % 2]) for i in range(layers)]}
+
+
 # --only design: Lomozen beside the dense model of the same width, depth, vocabulary and feed-forward
 # parameters per token (top * expert + shared = intermediate)
 DESIGN_SHAPES = {
@@ -86,6 +101,12 @@ DESIGN_SHAPES = {
 DUMAZEN_SHAPES = {
     "2k": (dumazen_shape(2048, 8, 16, 4608),) + DESIGN_SHAPES["2k"],
     "4k": (dumazen_shape(4096, 8, 32, 12288),) + DESIGN_SHAPES["4k"],
+}
+# --only design --design bozisun: Bozisun (6 layers of which two run twice: 8 layer runs) beside the dense model (the same
+# attention and feed-forward sizes) and Lomozen (routed experts of the same order), all of one width, depth and vocabulary
+BOZISUN_SHAPES = {
+    "2k": (bozisun_shape(2048, 6, 16, 3072, 32, 4, 768, (2, 4, 2)),) + DESIGN_SHAPES["2k"],
+    "4k": (bozisun_shape(4096, 6, 32, 8192, 64, 8, 1024, (2, 4, 2)),) + DESIGN_SHAPES["4k"],
 }
 PROMPT_LEN = 1024
 MAX_CONTEXT = 8192
@@ -212,6 +233,7 @@ def measure_design(args, rng):
 
     out = {"shape": args.design_shape, "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_prompt_len": PROMPT_LEN}
     models = (zip(("dumazen", "lomozen", "dense"), DUMAZEN_SHAPES[args.design_shape]) if args.design == "dumazen"
+              else zip(("bozisun", "lomozen", "dense"), BOZISUN_SHAPES[args.design_shape]) if args.design == "bozisun"
               else zip(("lomozen", "dense"), DESIGN_SHAPES[args.design_shape]))
     out["design"] = args.design
     for name, cfg in models:
@@ -220,7 +242,7 @@ def measure_design(args, rng):
         vocab = cfg.get("vocab") or cfg["vocab_size"]
         llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=16, max_num_seqs=32, max_model_len=4096,
                   num_blocks=1 + 32 * (2048 // 16) + 256, max_num_batched_tokens=PREFILL_TOKENS, enable_prefix_cache=False)
-        res = {"layers": len(llm.model.layers)}
+        res = {"layers": len(llm.model.layers), "layer_runs": len(llm.model.spec.schedule)}
         pre_s = measure_prefill(llm, rng, vocab)
         res["prefill_tokens_per_s"] = round(PREFILL_TOKENS / pre_s, 1)
         res["prefill_ms"] = round(pre_s * 1e3, 3)
@@ -231,7 +253,7 @@ def measure_design(args, rng):
         if not args.no_kernel_share:
             toks = rng.integers(0, vocab, size=PREFILL_TOKENS).tolist()
             llm.core.start_request("share")
-            res["prefill_kernels_us"] = kernel_times(lambda: llm.core.run([StepEntry("share", toks, [PREFILL_TOKENS - 1])]))
+            res["prefill_kernels_us"] = kernel_times(lambda: llm.core.run([StepEntry("share", toks, [PREFILL_TOKENS - 1])]), top=20)
             llm.core.finish_request("share")
             for _ in range(8):
                 llm.add_request(rng.integers(0, vocab, size=PROMPT_LEN).tolist(), SamplingParams(max_new_tokens=64))
@@ -239,7 +261,7 @@ def measure_design(args, rng):
                 llm.step()
             for _ in range(4):
                 llm.step()
-            res["decode_b8_kernels_us_8_steps"] = kernel_times(lambda: [llm.step() for _ in range(8)])
+            res["decode_b8_kernels_us_8_steps"] = kernel_times(lambda: [llm.step() for _ in range(8)], top=20)
             llm.abort_all()
         out[name] = res
         del llm
@@ -381,7 +403,7 @@ def main():
     ap.add_argument("--no-kernel-share", action="store_true", help="leave out the per-kernel time shares")
     ap.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k",
                     help="with --only design: the width of both models (2,048 or 4,096), 8 layers each")
-    ap.add_argument("--design", choices=["lomozen", "dumazen"], default="lomozen",
+    ap.add_argument("--design", choices=["lomozen", "dumazen", "bozisun"], default="lomozen",
                     help="with --only design: the architecture that is measured beside its kin of equal size")
     ap.add_argument("--design-models", default="", help="with --only design: only these of the models, with commas between them")
     ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt", "ttft", "calibrate", "design"], default=None,
