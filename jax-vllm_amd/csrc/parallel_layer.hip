@@ -30,6 +30,31 @@ embedding_pair_kernel(float* __restrict__ h, const T* __restrict__ table, const 
 // ---------------------------------------------------------------- two sublayers' outputs join the stream
 //   s = (ya + pa[0] + pa[1] + ...) + (yb + pb[0] + ...);   h += s;   out = T(h)  (if out)
 // ya, yb rows of the activation type or null; pa, pb float stacks of partial results or null.
+// V = 4: every pointer and stride allows 16-byte pieces of the float arrays (8 bytes of bfloat16).
+template <typename T, int V> struct PlVec { typedef T type __attribute__((ext_vector_type(V))); };
+template <typename T> struct PlVec<T, 1> { typedef T type; };
+template <typename T, int V>
+__device__ __forceinline__ void pl_load(const T* p, float (&v)[V]) {
+  if constexpr (V == 1) {
+    v[0] = to_f32(*p);
+  } else {
+    const typename PlVec<T, V>::type x = *(const typename PlVec<T, V>::type*)p;
+#pragma unroll
+    for (int e = 0; e < V; ++e) v[e] = to_f32<T>(x[e]);
+  }
+}
+template <typename T, int V>
+__device__ __forceinline__ void pl_store(T* p, const float (&v)[V]) {
+  if constexpr (V == 1) {
+    *p = from_f32<T>(v[0]);
+  } else {
+    typename PlVec<T, V>::type x;
+#pragma unroll
+    for (int e = 0; e < V; ++e) x[e] = from_f32<T>(v[e]);
+    *(typename PlVec<T, V>::type*)p = x;
+  }
+}
+
 template <typename T, int V>
 __global__ void __launch_bounds__(256)
 add_outputs_kernel(float* __restrict__ h, const T* __restrict__ ya, const float* __restrict__ pa, int na,
@@ -37,25 +62,26 @@ add_outputs_kernel(float* __restrict__ h, const T* __restrict__ ya, const float*
                    T* __restrict__ out, long long n) {
   const long long i0 = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * V;
   if (i0 >= n) return;
-  float a[V], b[V], x[V];
+  float a[V], b[V], x[V], t[V];
 #pragma unroll
-  for (int e = 0; e < V; ++e) {
-    a[e] = ya ? to_f32(ya[i0 + e]) : 0.f;
-    b[e] = yb ? to_f32(yb[i0 + e]) : 0.f;
-    x[e] = h[i0 + e];
+  for (int e = 0; e < V; ++e) a[e] = b[e] = 0.f;
+  pl_load<float, V>(h + i0, x);
+  if (ya) pl_load<T, V>(ya + i0, a);
+  if (yb) pl_load<T, V>(yb + i0, b);
+  for (int p = 0; p < na; ++p) {
+    pl_load<float, V>(pa + p * sa + i0, t);
+#pragma unroll
+    for (int e = 0; e < V; ++e) a[e] += t[e];
   }
-  for (int p = 0; p < na; ++p)
+  for (int p = 0; p < nb; ++p) {
+    pl_load<float, V>(pb + p * sb + i0, t);
 #pragma unroll
-    for (int e = 0; e < V; ++e) a[e] += pa[p * sa + i0 + e];
-  for (int p = 0; p < nb; ++p)
-#pragma unroll
-    for (int e = 0; e < V; ++e) b[e] += pb[p * sb + i0 + e];
-#pragma unroll
-  for (int e = 0; e < V; ++e) {
-    x[e] += a[e] + b[e];
-    h[i0 + e] = x[e];
-    if (out) out[i0 + e] = from_f32<T>(x[e]);
+    for (int e = 0; e < V; ++e) b[e] += t[e];
   }
+#pragma unroll
+  for (int e = 0; e < V; ++e) x[e] += a[e] + b[e];
+  pl_store<float, V>(h + i0, x);
+  if (out) pl_store<T, V>(out + i0, x);
 }
 
 // ---------------------------------------------------------------- gate of a per-layer token input
@@ -89,6 +115,27 @@ sigmoid_gate_heads_kernel(T* __restrict__ o, const T* __restrict__ g, long long 
   T* p = o + (t * heads + hd) * dp + e;
   const float gate = 1.f / (1.f + expf(-to_f32(g[t * ldg + r])));
   *p = from_f32<T>(to_f32(*p) * gate);
+}
+
+// The same with 16 bytes a lane, where the head sizes, the gate's row stride and both addresses allow it.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sigmoid_gate_heads_vec_kernel(T* __restrict__ o, const T* __restrict__ g, long long ldg, long long n, int heads, int dv,
+                              int dp) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T tv __attribute__((ext_vector_type(V)));
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long per = (long long)heads * dv / V;
+  if (i >= n * per) return;
+  const long long t = i / per;
+  const int r = (int)(i - t * per) * V;
+  const int hd = r / dv, e = r - hd * dv;
+  tv* p = (tv*)(o + (t * heads + hd) * dp + e);
+  const tv gv = *(const tv*)(g + t * ldg + r);
+  tv ov = *p;
+#pragma unroll
+  for (int k = 0; k < V; ++k) ov[k] = from_f32<T>(to_f32(ov[k]) / (1.f + expf(-to_f32(gv[k]))));
+  *p = ov;
 }
 
 // ---------------------------------------------------------------- soft cap on float logits
@@ -149,6 +196,13 @@ static int launch_add_outputs(float* h, const void* ya, const float* pa, int na,
     if (n <= 0 || heads <= 0 || dv <= 0) return 0;                                                                \
     if (dp < dv || ldg < (long long)heads * dv || (n * heads * dv + 255) / 256 > 0x7fffffffll)                    \
       return (int)hipErrorInvalidValue;                                                                           \
+    constexpr int V = 16 / (int)sizeof(T);                                                                        \
+    if (dv % V == 0 && dp % V == 0 && ldg % V == 0 && (uintptr_t)o % 16 == 0 && (uintptr_t)g % 16 == 0) {         \
+      const long long items = n * heads * dv / V;                                                                 \
+      hipLaunchKernelGGL(sigmoid_gate_heads_vec_kernel<T>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0,   \
+                         (hipStream_t)stream, (T*)o, (const T*)g, ldg, n, heads, dv, dp);                         \
+      return JV_LAUNCH_CHECK();                                                                                   \
+    }                                                                                                             \
     hipLaunchKernelGGL(sigmoid_gate_heads_kernel<T>, dim3((unsigned)((n * heads * dv + 255) / 256)), dim3(256),   \
                        0, (hipStream_t)stream, (T*)o, (const T*)g, ldg, n, heads, dv, dp);                        \
     return JV_LAUNCH_CHECK();                                                                                     \

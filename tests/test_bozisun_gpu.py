@@ -542,18 +542,23 @@ def test_kernel_router_with_a_bias_and_the_softmax_over_the_chosen(n):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-def test_kernel_attention_input_with_a_norm_per_head_and_a_wider_row(dtype):
+@pytest.mark.parametrize("shape", [(13, 12, 20, 32, 8, 17), (300, 32, 16, 48, 16, 24), (300, 128, 128, 128, 64, 512),
+                                   (300, 64, 64, 64, 64, 0), (260, 24, 8, 32, 0, 8)],
+                         ids=["few_odd", "many_padded", "many_128", "many_whole_rotation", "many_no_rotation"])
+def test_kernel_attention_input_with_a_norm_per_head_and_a_wider_row(dtype, shape):
+    """A wave a head for few tokens or odd sizes; 16 bytes a lane and the v heads through the tile writer for many."""
     from jax_vllm_amd.ops import kernels as K
 
     torch.manual_seed(5)
-    n, nq, nkv, dk, dv, dp, rd, ps, extra = 13, 4, 2, 12, 20, 32, 8, 8, 17
+    n, dk, dv, dp, rd, extra = shape
+    nq, nkv, ps = 4, 2, 8
     width = (nq + nkv) * dk + nkv * dv
     row = torch.randn(n, width + extra).to(dtype)
     qw, kw = torch.rand(dk) + 0.5, torch.rand(dk) + 0.5
     pos = torch.arange(n, dtype=torch.int32)
-    inv = 100.0 ** (-torch.arange(0, rd, 2, dtype=torch.float32) / rd)
-    table = K.rope_table(pos.cuda(), inv.cuda())
-    pages = 4
+    inv = 100.0 ** (-torch.arange(0, rd, 2, dtype=torch.float32) / max(rd, 1))
+    table = K.rope_table(pos.cuda(), inv.cuda()) if rd else None
+    pages = -(-n // ps) + 1
     kp = torch.zeros(pages + 1, nkv, ps, dp, dtype=dtype, device="cuda")
     vp = torch.zeros(pages + 1, nkv, dp, ps, dtype=dtype, device="cuda")
     slots = torch.tensor([(1 + t // ps) * ps + t % ps for t in range(n)], dtype=torch.int32)
@@ -561,14 +566,16 @@ def test_kernel_attention_input_with_a_norm_per_head_and_a_wider_row(dtype):
                             dp, norm_per_head=True)
     x = row.double()
     rot_cfg = {"dims": rd, "base": 100.0}
+    torch.cuda.synchronize()
     qq = P.rotate(P.rms_norm(x[:, :nq * dk].view(n, nq, dk), qw.double(), 1e-5), range(n), rot_cfg)
     kk = P.rotate(P.rms_norm(x[:, nq * dk:(nq + nkv) * dk].view(n, nkv, dk), kw.double(), 1e-5), range(n), rot_cfg)
     vv = x[:, (nq + nkv) * dk:width].view(n, nkv, dv)
-    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    tol = 1e-4 if dtype == torch.float32 else 4e-2      # float angles of positions up to 300 are off by 3e-5 themselves
     got = q.double().cpu().view(n, nq, dp)
-    assert float((got[:, :, :dk] - qq).abs().max()) < tol and float(got[:, :, dk:].abs().max()) == 0.0
+    assert float((got[:, :, :dk] - qq).abs().max()) < tol and (dp == dk or float(got[:, :, dk:].abs().max()) == 0.0)
+    kc, vc = kp.double().cpu(), vp.double().cpu()
     for t in range(n):
         page, s = 1 + t // ps, t % ps
-        assert float((kp[page, :, s, :dk].double().cpu() - kk[t]).abs().max()) < tol
-        assert float((vp[page, :, :dv, s].double().cpu() - vv[t]).abs().max()) < tol
-    assert float(kp[0].abs().max()) == 0.0 and float(kp[:, :, :, dk:].abs().max()) == 0.0
+        assert float((kc[page, :, s, :dk] - kk[t]).abs().max()) < tol
+        assert float((vc[page, :, :dv, s] - vv[t]).abs().max()) < tol
+    assert float(kc[0].abs().max()) == 0.0 and float(kc[:, :, :, dk:].abs().sum()) == 0.0 and float(vc[:, :, dv:].abs().sum()) == 0.0
