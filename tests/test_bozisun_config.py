@@ -70,7 +70,7 @@ def test_the_order_of_looped_layers():
         c = config(16, 20, [layer(attention(1, 1, 4, 4))] * n, loop=loop)
         return resolve(c)[1].layer_order()
 
-    assert order(6, (1, 3, 3)) == [0, 1, 2, 1, 2, 1, 2, 3, 4, 5]
+    assert order(5, (2, 4, 3)) == [0, 1, 2, 3, 2, 3, 2, 3, 4]
     assert order(3, None) == [0, 1, 2]
     assert order(3, (0, 3, 2)) == [0, 1, 2, 0, 1, 2]
     assert order(3, (2, 3, 1)) == [0, 1, 2]
@@ -120,7 +120,7 @@ def test_random_folder_is_read_back(tmp_path):
 def test_frequencies_of_the_rotation_part_follow_the_rescaling_rule():
     from jax_vllm_amd.parts.rotary import RotaryEncoding
 
-    for dims, base, sc in ((6, 100.0, YARN), (32, 1e6, dict(YARN, original=32)), (48, 50000.0, dict(YARN, original=1024, factor=8.0, fast=32.0)),
+    for dims, base, sc in ((6, 100.0, YARN), (32, 1e6, dict(YARN, original=32)), (48, 40000.0, dict(YARN, original=2048, factor=6.0, fast=16.0)),
                            (12, 500.0, None)):
         part = RotaryEncoding(dims + 4, base, dims, rescale=sc)
         want, amp = P.rotary_frequencies(rot(dims, base, sc))
@@ -128,9 +128,9 @@ def test_frequencies_of_the_rotation_part_follow_the_rescaling_rule():
         assert got.shape == (dims // 2,) and float(((got - want) / want).abs().max()) < 3e-7
         assert abs(part.amplitude - amp) < 1e-12
     # the three branches all occur: a pair that keeps its frequency, one slowed down by the factor, one blended
-    f = 50000.0 ** (-2.0 * torch.arange(24, dtype=torch.float64) / 48)
-    ratio = P.rotary_frequencies(rot(48, 50000.0, dict(YARN, original=1024, factor=8.0, fast=32.0)))[0] / f
-    assert float(ratio[0]) == 1.0 and abs(float(ratio[-1]) - 0.125) < 1e-12 and any(0.13 < float(r) < 0.99 for r in ratio)
+    f = 40000.0 ** (-2.0 * torch.arange(24, dtype=torch.float64) / 48)
+    ratio = P.rotary_frequencies(rot(48, 40000.0, dict(YARN, original=2048, factor=6.0, fast=16.0)))[0] / f
+    assert float(ratio[0]) == 1.0 and abs(float(ratio[-1]) - 1 / 6) < 1e-12 and any(0.18 < float(r) < 0.99 for r in ratio)
 
 
 def test_the_cache_manager_keeps_the_previous_token():

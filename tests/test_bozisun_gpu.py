@@ -420,7 +420,7 @@ def test_wider_layers_and_a_long_prompt(tmp_path, dtype):
         layer(attention(8, 2, 64, 64, scale=0.15, rot_=rot(32, 1e6)), None),
         layer(attention(2, 1, 128, 128, rot_=rot(64, 1e4, YARN)), moe(16, 4, 64)),
         layer(attention(4, 1, 48, 48), dense(192)),
-    ], bigram=(211, 31, 17), side=24, loop=(1, 4, 2), softcap=20.0))
+    ], bigram=(211, 31, 17), side=40, loop=(1, 4, 2), softcap=20.0))
     folder = make_folder(small, tmp_path)
     cfg, w = plain_of(folder)
     toks = tokens_of(cfg, 420, 9)
