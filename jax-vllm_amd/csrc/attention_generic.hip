@@ -8,6 +8,7 @@
 //   and sees keys j with  max(0, p - window + 1) <= j <= p   (window <= 0: all j <= p);
 //   key j lives in page block_tables[r, j / page_size] at slot j % page_size;
 //   q head h reads kv head h / (nq / nkv).
+// With `sinks` (one float per q head) every row's softmax denominator also holds exp(sinks[h]).
 // Cache layout: K pages[page][kv_head][slot][D], V pages[page][kv_head][D][slot].
 #include "common.h"
 
@@ -19,7 +20,8 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
                                const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                                const int* __restrict__ block_tables, int table_stride,
                                const int* __restrict__ token_req, const int* __restrict__ positions,
-                               int page_size, int nq, int nkv, int D, float scale, int window) {
+                               int page_size, int nq, int nkv, int D, float scale, int window,
+                               const float* __restrict__ sinks) {
   extern __shared__ float lds[];      // q[D] | p[64] | V offsets of the tile's keys as long long [64]
   float* qs = lds;
   float* ps = lds + D;
@@ -74,6 +76,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
       }
     }
   }
+  if (sinks) l += expf(sinks[h] - m);      // a term of the denominator that has no key and no value: exp(sink), unscaled
   const float inv_l = 1.f / l;
   T* o = out + t * (long long)nq * D + (long long)h * D;
 #pragma unroll
@@ -88,7 +91,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
       void* out, const void* q, long long q_row_stride, const void* k_pages, const void* v_pages,  \
       const int* block_tables, int table_stride, const int* token_req, const int* positions,       \
       int page_size, int n_tokens, int nq, int nkv, int D, float scale, int window,                \
-      void* stream) {                                                                              \
+      const float* sinks, void* stream) {                                                          \
     if (n_tokens <= 0) return 0;                                                                   \
     if (D > 64 * GEN_MAX_E || nkv <= 0 || nq % nkv != 0 || page_size <= 0)                         \
       return (int)hipErrorInvalidValue;                                                            \
@@ -96,7 +99,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
     hipLaunchKernelGGL(paged_attention_generic_kernel<T>, dim3(n_tokens, nq), dim3(64), shmem,     \
                        (hipStream_t)stream, (T*)out, (const T*)q, q_row_stride,                    \
                        (const T*)k_pages, (const T*)v_pages, block_tables, table_stride,           \
-                       token_req, positions, page_size, nq, nkv, D, scale, window);                \
+                       token_req, positions, page_size, nq, nkv, D, scale, window, sinks);         \
     return JV_LAUNCH_CHECK();                                                                      \
   }
 

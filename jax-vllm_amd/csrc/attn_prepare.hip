@@ -5,7 +5,8 @@
 //            or (per_head) over every head on its own, times a weight of dk elements shared by the heads, or none
 //            (a wave a (token, head))
 //   q, k  <- the first rot_dims elements of every head turned by the token's angles
-//   v     <- v * v_scale
+//   q     <- q * (1 + coef * ln(floor((position + 1) / every) + 1))    (optional: a query temperature that grows with position)
+//   v     <- v * v_scale;  the v heads begin at column v_off of the row (behind k, or AT k: values that are the keys as projected)
 // and stored in the layout the paged attention kernels read, every head padded with zeros to one size
 // Dp >= max(dk, dv): q rows [n][nq][Dp], key pages [pages][nkv][page_size][Dp], value pages transposed
 // [pages][nkv][Dp][page_size].  Zero padding leaves every score and every output element as it is; the
@@ -93,7 +94,8 @@ attn_prepare_heads_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long
                           const float* __restrict__ k_w, float eps, const float* __restrict__ cos_sin,
                           int rot_dims, const int* __restrict__ slot_mapping, T* __restrict__ k_pages,
                           T* __restrict__ v_pages, int page_size, int nq, int nkv, int dk, int dv, int dp,
-                          float v_scale, int v_elsewhere) {
+                          float v_scale, int v_elsewhere, long long v_off, const int* __restrict__ positions,
+                          float qt_coef, int qt_every) {
   extern __shared__ float heads_lds[];     // [4 waves][dk]
   const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE;
   float* buf = heads_lds + wid * dk;
@@ -109,7 +111,7 @@ attn_prepare_heads_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long
   const T* x = qkv + t * ld;
   if (is_v && store && !v_elsewhere) {
     const int kvh = head - nq - nkv;
-    const int c0 = (nq + nkv) * dk + kvh * dv;
+    const long long c0 = v_off + (long long)kvh * dv;
     T* dst = v_pages + (page * nkv + kvh) * (long long)dp * page_size + slot;
     for (int i = lane; i < dv; i += JV_WAVE)
       dst[(long long)i * page_size] = from_f32<T>((to_f32(x[c0 + i]) + (bias ? bias[c0 + i] : 0.f)) * v_scale);
@@ -129,6 +131,7 @@ attn_prepare_heads_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long
   }
   __syncthreads();      // every wave arrives once: the head in LDS is readable by the wave's other lanes
   if (!work) return;
+  const float temp = (is_q && positions) ? 1.f + qt_coef * logf((float)((positions[t] + 1) / qt_every) + 1.f) : 1.f;
   const int half = rot_dims / 2;
   T* dst = is_q ? q_out + (t * nq + head) * dp : k_pages + ((page * nkv + (head - nq)) * page_size + slot) * (long long)dp;
   for (int i = lane; i < (is_q ? dp : dk); i += JV_WAVE) {
@@ -143,7 +146,7 @@ attn_prepare_heads_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long
         val = i < half ? val * cs - other * sn : val * cs + other * sn;
       }
     }
-    dst[i] = from_f32<T>(val);
+    dst[i] = from_f32<T>(val * temp);
   }
 }
 
@@ -158,7 +161,7 @@ attn_prepare_heads_vec_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, 
                               const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
                               const float* __restrict__ cos_sin, int rot_dims, const int* __restrict__ slot_mapping,
                               T* __restrict__ k_pages, int page_size, long long n_items, int nq, int nkv, int dk,
-                              int dp, int lph) {
+                              int dp, int lph, const int* __restrict__ positions, float qt_coef, int qt_every) {
   constexpr int EP = 16 / (int)sizeof(T);
   typedef T tv __attribute__((ext_vector_type(EP)));
   const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE;
@@ -198,9 +201,10 @@ attn_prepare_heads_vec_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, 
     }
   }
   if (!live || !(is_q || store)) return;
+  const float temp = (is_q && positions) ? 1.f + qt_coef * logf((float)((positions[t] + 1) / qt_every) + 1.f) : 1.f;
   tv ov;
 #pragma unroll
-  for (int e = 0; e < EP; ++e) ov[e] = from_f32<T>(a[e]);
+  for (int e = 0; e < EP; ++e) ov[e] = from_f32<T>(a[e] * temp);
   if (is_q) {
     T* dst = q_out + (t * nq + head) * dp;
     *(tv*)(dst + e0) = ov;
@@ -221,15 +225,17 @@ attn_prepare_heads_vec_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, 
                                             const float* cos_sin, int rot_dims, const int* slot_mapping,        \
                                             void* k_pages, void* v_pages, int page_size, int n, int nq,         \
                                             int nkv, int dk, int dv, int dp, float v_scale, int per_head,       \
+                                            long long v_off, const int* positions, float qt_coef, int qt_every, \
                                             void* stream) {                                                     \
     if (n <= 0) return 0;                                                                                       \
+    if (v_off < 0 || (positions && (qt_every <= 0 || (q_w && !per_head)))) return (int)hipErrorInvalidValue;    \
+    if (q_w && !per_head && v_off != (long long)(nq + nkv) * dk) return (int)hipErrorInvalidValue;              \
     if (nq <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || dp < dk || dp < dv || rot_dims < 0 || rot_dims > dk ||     \
         rot_dims % 2 || (rot_dims && !cos_sin) || (!q_w) != (!k_w) || (slot_mapping && (!k_pages || !v_pages))) \
       return (int)hipErrorInvalidValue;                                                                         \
     if (!q_w || per_head) {                                                                                     \
       /* a wave a (token, head); the v heads of many tokens through the tile writer where its pieces align */  \
       constexpr int EP = 16 / (int)sizeof(T);                                                                   \
-      const long long v_off = (long long)(nq + nkv) * dk;                                                       \
       const bool v_tile = slot_mapping && !bias && v_written_by_tile<T>(k_pages, n, page_size, dv) &&           \
                           ld % EP == 0 && v_off % EP == 0 && ((uintptr_t)qkv % 16) == 0;                        \
       if (v_tile) {                                                                                             \
@@ -245,7 +251,8 @@ attn_prepare_heads_vec_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, 
         if (blocks > 0x7fffffffll) return (int)hipErrorInvalidValue;                                            \
         hipLaunchKernelGGL(attn_prepare_heads_vec_kernel<T>, dim3((unsigned)blocks), dim3(256), 0,              \
                            (hipStream_t)stream, (T*)q_out, (const T*)qkv, ld, q_w, k_w, eps, cos_sin, rot_dims, \
-                           slot_mapping, (T*)k_pages, page_size, items, nq, nkv, dk, dp, lph);                  \
+                           slot_mapping, (T*)k_pages, page_size, items, nq, nkv, dk, dp, lph, positions,        \
+                           qt_coef, qt_every);                                                                  \
         return JV_LAUNCH_CHECK();                                                                               \
       }                                                                                                         \
       const int walk = (v_tile || !slot_mapping) ? nq + nkv : nq + 2 * nkv;                                     \
@@ -253,7 +260,8 @@ attn_prepare_heads_vec_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, 
       hipLaunchKernelGGL(attn_prepare_heads_kernel<T>, dim3(n, (walk + 3) / 4), dim3(256),                      \
                          (size_t)4 * dk * sizeof(float), (hipStream_t)stream, (T*)q_out, (const T*)qkv, ld,     \
                          bias, q_w, k_w, eps, cos_sin, rot_dims, slot_mapping, (T*)k_pages, (T*)v_pages,        \
-                         page_size, nq, nkv, dk, dv, dp, v_scale, v_tile ? 1 : 0);                              \
+                         page_size, nq, nkv, dk, dv, dp, v_scale, v_tile ? 1 : 0, v_off, positions, qt_coef,   \
+                         qt_every);                                                                             \
       return JV_LAUNCH_CHECK();                                                                                 \
     }                                                                                                           \
     const size_t shmem = (size_t)(nq + nkv) * dk * sizeof(float);                                               \

@@ -57,9 +57,11 @@ __device__ __forceinline__ float jv_gated(int act, float gate, float up) {
 
 // Activations that stand alone (a feed-forward without a gate), in float; 0 means none.
 #define JV_ACT_GELU_ERF 3    // 0.5 z (1 + erf(z / sqrt(2)))
-__host__ __device__ __forceinline__ bool jv_plain_act_known(int act) { return act >= JV_ACT_SILU && act <= JV_ACT_GELU_ERF; }
+#define JV_ACT_TANH 4
+__host__ __device__ __forceinline__ bool jv_plain_act_known(int act) { return act >= JV_ACT_SILU && act <= JV_ACT_TANH; }
 __device__ __forceinline__ float jv_act(int act, float z) {
   if (act == JV_ACT_GELU_ERF) return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
+  if (act == JV_ACT_TANH) return tanhf(z);
   if (act == JV_ACT_GELU_TANH) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
   if (act == JV_ACT_SILU) return z / (1.f + expf(-z));
   return z;

@@ -35,11 +35,14 @@ extern "C" int jv_rope_table_amp(float* cos_sin, const int* positions, const flo
 //   cq[t]  = T( norm(q latent) * wq )
 //   e[t]   = [ T( norm(kv latent) * wkv ) | rotate(key part) ]  -> key page and transposed value page of the
 //            token's slot (slot_mapping[t] < 0: nothing is stored)
-// rotate: element i < half pairs with i + half (half = rot_dims / 2), elements from rot_dims on pass.
+// rotate: element i < half pairs with i + half (half = rot_dims / 2), or (interleaved) element 2i with 2i + 1,
+// both by the angle of frequency i; elements from rot_dims on pass.  q_rank may be 0 (queries that are projected
+// directly: no query latent, cq null); the kv latent begins at column kv_off of the row.
 // One block per token.
 template <typename T>
 __global__ void __launch_bounds__(256)
-latent_prepare_kernel(const T* __restrict__ proj, long long ld, int q_rank, int rank, int rot, int rot_dims,
+latent_prepare_kernel(const T* __restrict__ proj, long long ld, int q_rank, long long kv_off, int rank, int rot,
+                      int rot_dims, int interleaved,
                       const float* __restrict__ wq, const float* __restrict__ wkv, float eps,
                       const float* __restrict__ cos_sin, const int* __restrict__ slot_mapping,
                       T* __restrict__ cq, T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size) {
@@ -48,10 +51,10 @@ latent_prepare_kernel(const T* __restrict__ proj, long long ld, int q_rank, int 
   const T* x = proj + t * ld;
   float sq = 0.f, sk = 0.f;
   for (int c = threadIdx.x; c < q_rank; c += blockDim.x) { const float v = to_f32(x[c]); sq += v * v; }
-  for (int c = threadIdx.x; c < rank; c += blockDim.x) { const float v = to_f32(x[q_rank + c]); sk += v * v; }
-  sq = block_sum(sq, red);
+  for (int c = threadIdx.x; c < rank; c += blockDim.x) { const float v = to_f32(x[kv_off + c]); sk += v * v; }
+  if (q_rank) sq = block_sum(sq, red);
   sk = block_sum(sk, red);
-  const float inv_q = rsqrtf(sq / (float)q_rank + eps), inv_k = rsqrtf(sk / (float)rank + eps);
+  const float inv_q = q_rank ? rsqrtf(sq / (float)q_rank + eps) : 0.f, inv_k = rsqrtf(sk / (float)rank + eps);
   for (int c = threadIdx.x; c < q_rank; c += blockDim.x)
     cq[t * q_rank + c] = from_f32<T>(to_f32(x[c]) * inv_q * wq[c]);
   const long long slot = slot_mapping ? (long long)slot_mapping[t] : -1;
@@ -62,16 +65,21 @@ latent_prepare_kernel(const T* __restrict__ proj, long long ld, int q_rank, int 
   T* kd = k_pages + (page * page_size + off) * (long long)E;
   T* vd = v_pages + page * (long long)E * page_size + off;
   for (int c = threadIdx.x; c < rank; c += blockDim.x) {
-    const T v = from_f32<T>(to_f32(x[q_rank + c]) * inv_k * wkv[c]);
+    const T v = from_f32<T>(to_f32(x[kv_off + c]) * inv_k * wkv[c]);
     kd[c] = v;
     vd[(long long)c * page_size] = v;
   }
   const int half = rot_dims / 2;
-  const T* kr = x + q_rank + rank;
+  const T* kr = x + kv_off + rank;
   const float* cs = cos_sin + t * rot_dims;
   for (int c = threadIdx.x; c < rot; c += blockDim.x) {
     float v = to_f32(kr[c]);
-    if (c < half) v = v * cs[c] - to_f32(kr[c + half]) * cs[half + c];
+    if (interleaved) {
+      if (c < rot_dims) {
+        const int i = c >> 1;
+        v = (c & 1) ? v * cs[i] + to_f32(kr[c - 1]) * cs[half + i] : v * cs[i] - to_f32(kr[c + 1]) * cs[half + i];
+      }
+    } else if (c < half) v = v * cs[c] - to_f32(kr[c + half]) * cs[half + c];
     else if (c < rot_dims) v = v * cs[c - half] + to_f32(kr[c - half]) * cs[c];
     const T o = from_f32<T>(v);
     kd[rank + c] = o;
@@ -84,24 +92,29 @@ latent_prepare_kernel(const T* __restrict__ proj, long long ld, int q_rank, int 
 // One block per token.
 template <typename T>
 __global__ void __launch_bounds__(256)
-latent_query_rope_kernel(const T* __restrict__ q, T* __restrict__ qe, int heads, int dim, int rot, int rot_dims,
-                         int rank, const float* __restrict__ cos_sin) {
+latent_query_rope_kernel(const T* __restrict__ q, long long ldq, T* __restrict__ qe, int heads, int dim, int rot,
+                         int rot_dims, int rank, const float* __restrict__ cos_sin, int interleaved) {
   const long long t = blockIdx.x;
   const int half = rot_dims / 2;
   const float* cs = cos_sin + t * rot_dims;
   for (int i = threadIdx.x; i < heads * rot; i += blockDim.x) {
     const int h = i / rot, c = i - h * rot;
-    const T* x = q + (t * heads + h) * (long long)(dim + rot) + dim;
+    const T* x = q + t * ldq + h * (long long)(dim + rot) + dim;
     float v = to_f32(x[c]);
-    if (c < half) v = v * cs[c] - to_f32(x[c + half]) * cs[half + c];
+    if (interleaved) {
+      if (c < rot_dims) {
+        const int i2 = c >> 1;
+        v = (c & 1) ? v * cs[i2] + to_f32(x[c - 1]) * cs[half + i2] : v * cs[i2] - to_f32(x[c + 1]) * cs[half + i2];
+      }
+    } else if (c < half) v = v * cs[c] - to_f32(x[c + half]) * cs[half + c];
     else if (c < rot_dims) v = v * cs[c - half] + to_f32(x[c - half]) * cs[c];
     qe[(t * heads + h) * (long long)(rank + rot) + rank + c] = from_f32<T>(v);
   }
 }
 
 // ---------------------------------------------------------------- one small matrix per head
-//   y[t, h * ys + n] = ( sum_k W[h][n][k] * x[t * ldx + h * xs + k] ) * ( g ? sigmoid(g[t * ldg + h * N + n]) : 1 )
-// for n < N, k < K.  Float accumulation in ascending k whatever the batch.  64 x 64 outputs a block of 256
+//   y[t, h * ys + n] = ( sum_k W[h][n][k] * x[t * ldx + h * xs + k] ) * ( g ? sigmoid(g[t * ldg + h * gn + (gn > 1 ? n : 0)]) : 1 )
+// for n < N, k < K; gn = N: a gate per output element, gn = 1: one gate for all of a head's outputs.  Float accumulation in ascending k whatever the batch.  64 x 64 outputs a block of 256
 // threads, k in slabs of 16 through LDS; blockIdx.z is the head.
 #define HL_BM 64
 #define HL_BN 64
@@ -109,7 +122,7 @@ latent_query_rope_kernel(const T* __restrict__ q, T* __restrict__ qe, int heads,
 template <typename T>
 __global__ void __launch_bounds__(256)
 head_linear_kernel(T* __restrict__ y, long long ldy, int ys, const T* __restrict__ x, long long ldx, int xs,
-                   const T* __restrict__ W, int M, int N, int K, const T* __restrict__ g, long long ldg) {
+                   const T* __restrict__ W, int M, int N, int K, const T* __restrict__ g, long long ldg, int gn) {
   __shared__ float As[HL_BK][HL_BM + 4];
   __shared__ float Ws[HL_BK][HL_BN + 4];
   const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
@@ -150,7 +163,7 @@ head_linear_kernel(T* __restrict__ y, long long ldy, int ys, const T* __restrict
       const int n = n0 + tx * 4 + j;
       if (n >= N) continue;
       float v = acc[i][j];
-      if (g) v *= 1.f / (1.f + expf(-to_f32(g[(long long)m * ldg + (long long)h * N + n])));
+      if (g) v *= 1.f / (1.f + expf(-to_f32(g[(long long)m * ldg + (long long)h * gn + (gn > 1 ? n : 0)])));
       y[(long long)m * ldy + (long long)h * ys + n] = from_f32<T>(v);
     }
   }
@@ -163,7 +176,7 @@ head_linear_kernel(T* __restrict__ y, long long ldy, int ys, const T* __restrict
 template <typename T>
 __global__ void __launch_bounds__(256)
 head_linear_rows_kernel(T* __restrict__ y, long long ldy, int ys, const T* __restrict__ x, long long ldx, int xs,
-                        const T* __restrict__ W, int M, int N, int K, const T* __restrict__ g, long long ldg) {
+                        const T* __restrict__ W, int M, int N, int K, const T* __restrict__ g, long long ldg, int gn) {
   extern __shared__ float hl[];          // x [M][K] | partial sums [4][HL_ROWS][64]
   float* xr = hl;
   float* red = hl + M * K;
@@ -201,7 +214,7 @@ head_linear_rows_kernel(T* __restrict__ y, long long ldy, int ys, const T* __res
     float v = 0.f;
 #pragma unroll
     for (int p = 0; p < 4; ++p) v += red[(p * HL_ROWS + t) * 64 + (threadIdx.x & 63)];
-    if (g) v *= 1.f / (1.f + expf(-to_f32(g[(long long)t * ldg + (long long)h * N + n])));
+    if (g) v *= 1.f / (1.f + expf(-to_f32(g[(long long)t * ldg + (long long)h * gn + (gn > 1 ? n : 0)])));
     y[(long long)t * ldy + (long long)h * ys + n] = from_f32<T>(v);
   }
 }
@@ -215,7 +228,7 @@ typedef float hl_f32x4 __attribute__((ext_vector_type(4)));
 __global__ void __launch_bounds__(256)
 head_linear_mfma_kernel(bf16_t* __restrict__ y, long long ldy, int ys, const bf16_t* __restrict__ x, long long ldx,
                         int xs, const bf16_t* __restrict__ W, int M, int N, int K, const bf16_t* __restrict__ g,
-                        long long ldg) {
+                        long long ldg, int gn) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 15, lc = lane >> 4;
   const int h = blockIdx.z, n0 = blockIdx.x * 16, m0 = (blockIdx.y * 4 + wave) * 16;
   if (m0 >= M) return;
@@ -237,59 +250,66 @@ head_linear_mfma_kernel(bf16_t* __restrict__ y, long long ldy, int ys, const bf1
     const int n = nb + e;
     if (n >= N) continue;
     float v = acc[e];
-    if (g) v *= 1.f / (1.f + expf(-(float)g[(long long)m * ldg + (long long)h * N + n]));
+    if (g) v *= 1.f / (1.f + expf(-(float)g[(long long)m * ldg + (long long)h * gn + (gn > 1 ? n : 0)]));
     y[(long long)m * ldy + (long long)h * ys + n] = (bf16_t)v;
   }
 }
 
 extern "C" int jv_head_linear_mfma_bf16(void* y, long long ldy, int ys, const void* x, long long ldx, int xs,
                                         const void* W, int M, int N, int K, int heads, const void* g, long long ldg,
-                                        void* stream) {
+                                        int gn, void* stream) {
   if (M <= 0 || N <= 0 || heads <= 0) return 0;
+  if (g && gn != N && gn != 1) return (int)hipErrorInvalidValue;
   const unsigned gy = (M + 63) / 64;
   if (gy > 65535u || heads > 65535 || K < 8 || K % 8 || ldx % 8 || xs % 8) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(head_linear_mfma_kernel, dim3((N + 15) / 16, gy, heads), dim3(256), 0, (hipStream_t)stream,
-                     (bf16_t*)y, ldy, ys, (const bf16_t*)x, ldx, xs, (const bf16_t*)W, M, N, K, (const bf16_t*)g, ldg);
+                     (bf16_t*)y, ldy, ys, (const bf16_t*)x, ldx, xs, (const bf16_t*)W, M, N, K, (const bf16_t*)g, ldg, gn);
   return JV_LAUNCH_CHECK();
 }
 
 #define DEFINE_LATENT(SUF, T)                                                                              \
-  extern "C" int jv_latent_prepare_##SUF(const void* proj, long long ld, int n, int q_rank, int rank,      \
-                                         int rot, int rot_dims, const float* wq, const float* wkv,         \
+  extern "C" int jv_latent_prepare_##SUF(const void* proj, long long ld, int n, int q_rank, long long kv_off, \
+                                         int rank,                                                         \
+                                         int rot, int rot_dims, int interleaved, const float* wq,          \
+                                         const float* wkv,                                                 \
                                          float eps, const float* cos_sin, const int* slot_mapping,         \
                                          void* cq, void* k_pages, void* v_pages, int page_size,            \
                                          void* stream) {                                                   \
     if (n <= 0) return 0;                                                                                  \
-    if (q_rank <= 0 || rank <= 0 || rot < 0 || rot_dims < 0 || rot_dims > rot || rot_dims % 2)             \
+    if (q_rank < 0 || kv_off < 0 || rank <= 0 || rot < 0 || rot_dims < 0 || rot_dims > rot || rot_dims % 2 || \
+        (q_rank && (!wq || !cq)))                                                                          \
       return (int)hipErrorInvalidValue;                                                                    \
     hipLaunchKernelGGL(latent_prepare_kernel<T>, dim3(n), dim3(256), 0, (hipStream_t)stream,               \
-                       (const T*)proj, ld, q_rank, rank, rot, rot_dims, wq, wkv, eps, cos_sin,             \
+                       (const T*)proj, ld, q_rank, kv_off, rank, rot, rot_dims, interleaved, wq, wkv, eps, cos_sin, \
                        slot_mapping, (T*)cq, (T*)k_pages, (T*)v_pages, page_size);                         \
     return JV_LAUNCH_CHECK();                                                                              \
   }                                                                                                        \
-  extern "C" int jv_latent_query_rope_##SUF(const void* q, void* qe, int n, int heads, int dim, int rot,   \
-                                            int rot_dims, int rank, const float* cos_sin, void* stream) {  \
+  extern "C" int jv_latent_query_rope_##SUF(const void* q, long long ldq, void* qe, int n, int heads, int dim, \
+                                            int rot,                                                       \
+                                            int rot_dims, int rank, const float* cos_sin, int interleaved, \
+                                            void* stream) {                                                \
     if (n <= 0 || heads * rot <= 0) return 0;                                                              \
     if (rot_dims > rot || rot_dims % 2) return (int)hipErrorInvalidValue;                                  \
     hipLaunchKernelGGL(latent_query_rope_kernel<T>, dim3(n), dim3(256), 0, (hipStream_t)stream,            \
-                       (const T*)q, (T*)qe, heads, dim, rot, rot_dims, rank, cos_sin);                     \
+                       (const T*)q, ldq, (T*)qe, heads, dim, rot, rot_dims, rank, cos_sin, interleaved);   \
     return JV_LAUNCH_CHECK();                                                                              \
   }                                                                                                        \
   extern "C" int jv_head_linear_##SUF(void* y, long long ldy, int ys, const void* x, long long ldx,        \
                                       int xs, const void* W, int M, int N, int K, int heads,               \
-                                      const void* g, long long ldg, void* stream) {                        \
+                                      const void* g, long long ldg, int gn, void* stream) {                \
     if (M <= 0 || N <= 0 || heads <= 0) return 0;                                                          \
+    if (g && gn != N && gn != 1) return (int)hipErrorInvalidValue;                                         \
     const unsigned gy = (M + HL_BM - 1) / HL_BM;                                                           \
     if (gy > 65535u || heads > 65535 || K < 0) return (int)hipErrorInvalidValue;                           \
     if (M <= HL_ROWS && K > 0 && (size_t)(M * K + 4 * HL_ROWS * 64) * sizeof(float) <= 60 * 1024) {        \
       hipLaunchKernelGGL(head_linear_rows_kernel<T>, dim3((N + 63) / 64, heads), dim3(256),                \
                          (size_t)(M * K + 4 * HL_ROWS * 64) * sizeof(float), (hipStream_t)stream, (T*)y,   \
-                         ldy, ys, (const T*)x, ldx, xs, (const T*)W, M, N, K, (const T*)g, ldg);           \
+                         ldy, ys, (const T*)x, ldx, xs, (const T*)W, M, N, K, (const T*)g, ldg, gn);       \
       return JV_LAUNCH_CHECK();                                                                            \
     }                                                                                                      \
     hipLaunchKernelGGL(head_linear_kernel<T>, dim3((N + HL_BN - 1) / HL_BN, gy, heads), dim3(256), 0,      \
                        (hipStream_t)stream, (T*)y, ldy, ys, (const T*)x, ldx, xs, (const T*)W, M, N, K,    \
-                       (const T*)g, ldg);                                                                  \
+                       (const T*)g, ldg, gn);                                                              \
     return JV_LAUNCH_CHECK();                                                                              \
   }
 

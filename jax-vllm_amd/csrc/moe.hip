@@ -3,7 +3,9 @@
 // known only on the device, so every launch is sized by upper bounds and blocks without work leave.
 //
 //   route:   z = router logits (float, plus an optional bias per expert) -> the `top` largest per token
-//            (lowest index among equals), weight = sigmoid(z), or the softmax over the chosen logits alone
+//            (lowest index among equals), weight = sigmoid(z), or the softmax over the chosen logits alone, or
+//            ("sigmoid_normed") the largest sigmoid(z) + correction chosen, weight = sigmoid(z) over the sum of the
+//            chosen sigmoids (+ 1e-20) times a constant
 //   group:   entry s = token * top + kk  ->  position in a list ordered by expert; tiles of MOE_TM rows
 //            that never straddle two experts
 //   gate/up: z[pos] = act(w g) * (w u),  g = Wg[e] x[token], u = Wu[e] x[token]      (w = the entry's weight
@@ -21,13 +23,18 @@
 // logits (a copy in LDS), the wave agrees on the best, and the lane that scans the chosen expert takes it out.
 #define MOE_SCORE_SIGMOID 0          // weight = sigmoid(logit)
 #define MOE_SCORE_SOFTMAX_CHOSEN 1   // weight = exp(logit) / sum of exp over the token's chosen logits
+#define MOE_SCORE_SIGMOID_NORMED 2   // chosen by sigmoid(logit) + correction; weight = sigmoid(logit) / (sum over the chosen + 1e-20) * scale
 __device__ __forceinline__ void moe_pick(float* zt, int experts, int top, int lane, int* ids, float* weights,
-                                         int score) {
+                                         int score, const float* __restrict__ correction = nullptr,
+                                         float weight_scale = 1.f) {
+  const bool normed = score == MOE_SCORE_SIGMOID_NORMED;
   for (int kk = 0; kk < top; ++kk) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int e = lane; e < experts; e += JV_WAVE) {
-      const float v = zt[e];
+      float v = zt[e];
+      // an expert already taken holds -inf and stays out; the others compete with their corrected sigmoid
+      if (normed && v != -INFINITY) v = 1.f / (1.f + expf(-v)) + (correction ? correction[e] : 0.f);
       if (v > bv || (bi == 0x7fffffff && v == v)) { bv = v; bi = e; }
     }
 #pragma unroll
@@ -39,7 +46,8 @@ __device__ __forceinline__ void moe_pick(float* zt, int experts, int top, int la
     if (bi == 0x7fffffff) { bi = kk; bv = __builtin_nanf(""); }      // a row of NaN: some expert, the NaN shows in the output
     if (lane == 0) {
       ids[kk] = bi;
-      weights[kk] = score == MOE_SCORE_SOFTMAX_CHOSEN ? bv : 1.f / (1.f + expf(-bv));
+      const float z = normed ? zt[bi] : bv;          // the logit itself: the correction takes part in the choice only
+      weights[kk] = score == MOE_SCORE_SOFTMAX_CHOSEN ? bv : 1.f / (1.f + expf(-z));
     }
     if ((bi & (JV_WAVE - 1)) == lane) zt[bi] = -INFINITY;
   }
@@ -55,19 +63,26 @@ __device__ __forceinline__ void moe_pick(float* zt, int experts, int top, int la
     const float inv = 1.f / sum;
     for (int kk = 0; kk < top; ++kk) weights[kk] *= inv;
   }
+  if (normed && lane == 0) {
+    float sum = 0.f;
+    for (int kk = 0; kk < top; ++kk) sum += weights[kk];
+    const float f = weight_scale / (sum + 1e-20f);
+    for (int kk = 0; kk < top; ++kk) weights[kk] *= f;
+  }
 }
 
 // a wave per token, 4 tokens a block
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int n, int experts, int top,
-                 int score, int* __restrict__ ids, float* __restrict__ weights) {
+                 int score, int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ correction,
+                 float weight_scale) {
   extern __shared__ float zs[];      // [4][experts]
   const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE;
   const long long t = (long long)blockIdx.x * 4 + wid;
   if (t >= n) return;
   float* zt = zs + wid * experts;
   for (int e = lane; e < experts; e += JV_WAVE) zt[e] = logits[t * experts + e] + (bias ? bias[e] : 0.f);
-  moe_pick(zt, experts, top, lane, ids + t * top, weights + t * top, score);
+  moe_pick(zt, experts, top, lane, ids + t * top, weights + t * top, score, correction, weight_scale);
 }
 
 // Router and choice in one launch: a block takes up to MOE_RT tokens, their rows in LDS as floats; a wave per
@@ -80,7 +95,7 @@ template <typename T>
 __global__ void __launch_bounds__(1024)
 moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, const float* __restrict__ bias, int n, int hidden,
                   int experts, int top, int tb, int score, int* __restrict__ ids, float* __restrict__ weights,
-                  float* __restrict__ logits_out) {
+                  float* __restrict__ logits_out, const float* __restrict__ correction, float weight_scale) {
   extern __shared__ float rs[];      // x [tb][hidden] | z [tb][experts]
   float* xs = rs;
   float* z = rs + tb * hidden;
@@ -127,7 +142,8 @@ moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, const float*
   }
   __syncthreads();
   for (int t = wid; t < nt; t += nw)
-    moe_pick(z + t * experts, experts, top, lane, ids + (t0 + t) * top, weights + (t0 + t) * top, score);
+    moe_pick(z + t * experts, experts, top, lane, ids + (t0 + t) * top, weights + (t0 + t) * top, score, correction,
+             weight_scale);
 }
 
 // One block.  meta: [0] number of tiles; offsets [experts + 1]; tile_expert / tile_row0 [max_tiles];
@@ -295,16 +311,28 @@ moe_down_kernel(float* __restrict__ y, const T* __restrict__ z, const T* __restr
   }
 }
 
+// A share of every token that carries a gate of the token's own: out[t][c] = float(y[t][c]) * sigmoid(g[t * ldg])
+// (a shared expert that joins the chosen experts' float stack under one number per token).
+template <typename T>
+__global__ void __launch_bounds__(256)
+row_gate_kernel(float* __restrict__ out, const T* __restrict__ y, const T* __restrict__ g, long long ldg, long long n,
+                int hidden) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * hidden) return;
+  const long long t = i / hidden;
+  out[i] = to_f32(y[i]) / (1.f + expf(-to_f32(g[t * ldg])));
+}
+
 extern "C" int jv_moe_tile_rows() { return MOE_TM; }
 
 extern "C" int jv_moe_route(const float* logits, const float* bias, int n, int experts, int top, int score, int* ids,
-                            float* weights, void* stream) {
+                            float* weights, const float* correction, float weight_scale, void* stream) {
   if (n <= 0) return 0;
-  if (experts <= 0 || top <= 0 || top > experts || score < 0 || score > MOE_SCORE_SOFTMAX_CHOSEN)
+  if (experts <= 0 || top <= 0 || top > experts || score < 0 || score > MOE_SCORE_SIGMOID_NORMED)
     return (int)hipErrorInvalidValue;
   if (experts > 3840) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(moe_route_kernel, dim3((n + 3) / 4), dim3(256), 4 * experts * sizeof(float), (hipStream_t)stream,
-                     logits, bias, n, experts, top, score, ids, weights);
+                     logits, bias, n, experts, top, score, ids, weights, correction, weight_scale);
   return JV_LAUNCH_CHECK();
 }
 
@@ -320,17 +348,27 @@ extern "C" int jv_moe_group(const int* ids, int entries, int experts, int tile_r
 #define DEFINE_MOE(SUF, T)                                                                                        \
   extern "C" int jv_moe_router_##SUF(const void* x, const void* W, const float* bias, int n, int hidden,          \
                                      int experts, int top, int score, int* ids, float* weights,                   \
-                                     float* logits_out, void* stream) {                                           \
+                                     float* logits_out, const float* correction, float weight_scale,              \
+                                     void* stream) {                                                              \
     if (n <= 0) return 0;                                                                                         \
     if (experts <= 0 || top <= 0 || top > experts || hidden <= 0 || (hidden + experts) > 15000 || score < 0 ||    \
-        score > MOE_SCORE_SOFTMAX_CHOSEN)                                                                         \
+        score > MOE_SCORE_SIGMOID_NORMED)                                                                         \
       return (int)hipErrorInvalidValue;                                                                           \
     int tb = 15000 / (hidden + experts);             /* tokens of a block: their rows and logits in 60 KB */      \
     tb = tb > MOE_RT ? MOE_RT : tb;                                                                               \
     while (tb > 1 && (n + tb - 1) / tb < 128) --tb;  /* few tokens: more blocks rather than rows sharing a read */ \
     hipLaunchKernelGGL(moe_router_kernel<T>, dim3((n + tb - 1) / tb), dim3(1024),                                  \
                        (size_t)tb * (hidden + experts) * sizeof(float), (hipStream_t)stream, (const T*)x,         \
-                       (const T*)W, bias, n, hidden, experts, top, tb, score, ids, weights, logits_out);          \
+                       (const T*)W, bias, n, hidden, experts, top, tb, score, ids, weights, logits_out,           \
+                       correction, weight_scale);                                                                 \
+    return JV_LAUNCH_CHECK();                                                                                     \
+  }                                                                                                               \
+  extern "C" int jv_row_gate_##SUF(float* out, const void* y, const void* g, long long ldg, long long n,         \
+                                   int hidden, void* stream) {                                                    \
+    if (n <= 0 || hidden <= 0) return 0;                                                                          \
+    if ((n * hidden + 255) / 256 > 0x7fffffffll) return (int)hipErrorInvalidValue;                                \
+    hipLaunchKernelGGL(row_gate_kernel<T>, dim3((unsigned)((n * hidden + 255) / 256)), dim3(256), 0,              \
+                       (hipStream_t)stream, out, (const T*)y, (const T*)g, ldg, n, hidden);                       \
     return JV_LAUNCH_CHECK();                                                                                     \
   }                                                                                                               \
   extern "C" int jv_moe_gate_up_##SUF(void* z, const void* x, const void* Wg, const void* Wu, const int* meta,    \

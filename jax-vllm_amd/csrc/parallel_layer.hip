@@ -12,17 +12,17 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 embedding_pair_kernel(float* __restrict__ h, const T* __restrict__ table, const T* __restrict__ pair,
                       const int* __restrict__ ids, const int* __restrict__ prev, int hidden, int rows,
-                      long long buckets, long long mul_prev, long long mul_cur) {
+                      long long buckets, long long mul_prev, long long mul_cur, float scale) {
   const long long t = blockIdx.x;
   const int id = ids[t], pv = prev[t];
   const bool inside = id >= 0 && id < rows && pv < rows;
   const long long r = pv < 0 ? buckets : (((long long)pv * mul_prev + (long long)id * mul_cur) % buckets);
   const T* a = table + (long long)(inside ? id : 0) * hidden;
-  const T* b = pair + (inside ? r : 0) * hidden;
+  const T* b = pair ? pair + (inside ? r : 0) * hidden : nullptr;     // no second table: the scaled row alone
   float* out = h + t * hidden;
   const float nan = __builtin_nanf("");
   for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-    const float v = to_f32(a[c]) + to_f32(b[c]);
+    const float v = to_f32(a[c]) * scale + (b ? to_f32(b[c]) : 0.f);
     out[c] = inside ? v : nan;
   }
 }
@@ -164,12 +164,12 @@ static int launch_add_outputs(float* h, const void* ya, const float* pa, int na,
 #define DEFINE_PARALLEL_LAYER(SUF, T)                                                                             \
   extern "C" int jv_embedding_pair_##SUF(float* h, const void* table, const void* pair, const int* ids,           \
                                          const int* prev, int n_tokens, int hidden, int rows, long long buckets,  \
-                                         long long mul_prev, long long mul_cur, void* stream) {                   \
+                                         long long mul_prev, long long mul_cur, float scale, void* stream) {      \
     if (n_tokens <= 0) return 0;                                                                                  \
     if (buckets <= 0 || mul_prev < 0 || mul_cur < 0 || mul_prev > 0x7fffffffll || mul_cur > 0x7fffffffll)         \
       return (int)hipErrorInvalidValue;                                                                           \
     hipLaunchKernelGGL(embedding_pair_kernel<T>, dim3(n_tokens), dim3(256), 0, (hipStream_t)stream, h,            \
-                       (const T*)table, (const T*)pair, ids, prev, hidden, rows, buckets, mul_prev, mul_cur);     \
+                       (const T*)table, (const T*)pair, ids, prev, hidden, rows, buckets, mul_prev, mul_cur, scale); \
     return JV_LAUNCH_CHECK();                                                                                     \
   }                                                                                                               \
   /* n = rows * hidden elements; the stacks' strides in elements; `vec`: every pointer and stride allows 4 */    \

@@ -7,6 +7,7 @@
 // Row r = rows ? rows[i] : i.
 //   v   = (y ? y[r] : 0) + parts[0][r] + parts[1][r] + ... (+ bias)   (the sublayer's output; parts added in order)
 //   x   = h[r] + v * rsqrt(mean(v^2) + eps) * wb                 (float)
+//         or, where wb is null (a sublayer's output that joins the stream under a constant only), h[r] + v * plain_scale
 //   if (!rows) h[r] = x
 //   if (out)   out[i] = T( x * rsqrt(mean(x^2) + eps_out) * w ),   or T(x) where w is null
 // One block per output row; the row is kept in LDS between the passes (hidden floats).
@@ -16,7 +17,7 @@ postnorm_add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ y, cons
                             int n_parts, long long part_stride, const float* __restrict__ bias,
                             const float* __restrict__ wb,
                             const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
-                            int hidden, float eps, float eps_out) {
+                            int hidden, float eps, float eps_out, float plain_scale) {
   extern __shared__ float row[];
   __shared__ float red[32];
   const long long i = blockIdx.x;
@@ -31,10 +32,10 @@ postnorm_add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ y, cons
     ss += v * v;
   }
   ss = block_sum(ss, red);
-  const float inv_b = rsqrtf(ss / (float)hidden + eps);
+  const float inv_b = wb ? rsqrtf(ss / (float)hidden + eps) : plain_scale;
   float ss2 = 0.f;
   for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-    const float x = hr[c] + row[c] * inv_b * wb[c];
+    const float x = hr[c] + row[c] * inv_b * (wb ? wb[c] : 1.f);
     if (!rows) hr[c] = x;
     row[c] = x;
     ss2 += x * x;
@@ -94,7 +95,7 @@ postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, 
                                 int n_parts, long long part_stride, const float* __restrict__ bias,
                                 const float* __restrict__ wb,
                                 const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
-                                int hidden, float eps, float eps_out) {
+                                int hidden, float eps, float eps_out, float plain_scale) {
   __shared__ float red[32];
   const long long i = blockIdx.x;
   const long long r = rows ? (long long)rows[i] : i;
@@ -106,7 +107,7 @@ postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, 
     const int cc = c < hidden ? c : 0;           // a piece beyond the row reads the row's first piece, its share is left out
     v[q] = y ? sn_load4<T>(y + r * hidden + cc) : float4{0.f, 0.f, 0.f, 0.f};
     x[q] = *(const float4*)(h + r * hidden + cc);
-    b[q] = *(const float4*)(wb + cc);
+    b[q] = wb ? *(const float4*)(wb + cc) : float4{1.f, 1.f, 1.f, 1.f};
   }
   for (int p = 0; p < n_parts; ++p) {
 #pragma unroll
@@ -128,7 +129,7 @@ postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, 
   for (int q = 0; q < SN_V; ++q)
     if ((threadIdx.x + q * 256) * 4 < hidden) ss += v[q].x * v[q].x + v[q].y * v[q].y + v[q].z * v[q].z + v[q].w * v[q].w;
   ss = block_sum(ss, red);
-  const float inv_b = rsqrtf(ss / (float)hidden + eps);
+  const float inv_b = wb ? rsqrtf(ss / (float)hidden + eps) : plain_scale;
   float ss2 = 0.f;
 #pragma unroll
   for (int q = 0; q < SN_V; ++q) {
@@ -166,19 +167,20 @@ postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, 
                                                long long part_stride, const float* bias,               \
                                                const float* wb, const float* w,                         \
                                                void* out, const int* rows, int n_out, int hidden,        \
-                                               float eps, float eps_out, void* stream) {                 \
+                                               float eps, float eps_out, float plain_scale,              \
+                                               void* stream) {                                           \
     if (n_out <= 0 || hidden <= 0) return 0;                                                             \
     if ((!y && n_parts <= 0) || hidden > 16384) return (int)hipErrorInvalidValue;                        \
     if (hidden % 4 == 0 && hidden <= 4 * SN_V * 256) {                                                   \
       hipLaunchKernelGGL(postnorm_add_rmsnorm_vec_kernel<T>, dim3(n_out), dim3(256), 0,                  \
                          (hipStream_t)stream, h, (const T*)y, parts, n_parts, part_stride, bias, wb, w,  \
-                         (T*)out, rows, hidden, eps, eps_out);                                           \
+                         (T*)out, rows, hidden, eps, eps_out, plain_scale);                              \
       return JV_LAUNCH_CHECK();                                                                          \
     }                                                                                                    \
     hipLaunchKernelGGL(postnorm_add_rmsnorm_kernel<T>, dim3(n_out), dim3(256), hidden * sizeof(float),   \
                        (hipStream_t)stream, h, (const T*)y, parts, n_parts, part_stride, bias, wb, w,    \
                        (T*)out,                                                                          \
-                       rows, hidden, eps, eps_out);                                                      \
+                       rows, hidden, eps, eps_out, plain_scale);                                         \
     return JV_LAUNCH_CHECK();                                                                            \
   }                                                                                                      \
   extern "C" int jv_gated_rmsnorm_##SUF(void* out, const float* o, const void* g, long long g_stride,    \

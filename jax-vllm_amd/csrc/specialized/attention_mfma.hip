@@ -77,6 +77,7 @@ struct AttnArgs {
   int page_size, page_shift, nq, nkv;   // page_shift: log2(page_size) or -1
   float scale_log2;           // softmax scale * log2(e)
   int window;                 // <= 0: none
+  const float* sinks;         // [nq] or null: exp(sinks[h]) joins every row's softmax denominator (no key, no value, unscaled)
   // decode only
   int num_splits;
   float* part_acc;            // [n_work, nq, num_splits, D]
@@ -477,6 +478,7 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
     float l = l_lane[t] + __shfl_xor(l_lane[t], 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (row_ok[t]) {
+      if (p.sinks) l += fast_exp2(p.sinks[g * G + hg[t]] * 1.4426950408889634f - m_ref[t] * p.scale_log2);
       const float inv = 1.f / l;
       bf16_t* o = p.out + (long long)(q_start + qi[t]) * p.nq * D + (long long)(g * G + hg[t]) * D + lc * 4;
 #pragma unroll
@@ -1083,6 +1085,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
   float l = l_lane + __shfl_xor(l_lane, 32, 64);
   if (row_ok) {
+    if (p.sinks) l += fast_exp2(p.sinks[g * G + hg] * 1.4426950408889634f - m_ref * p.scale_log2);
     const float inv = 1.f / l;
     bf16_t* o = p.out + (long long)(q_start + qi) * p.nq * D + (long long)(g * G + hg) * D + h * 4;
 #pragma unroll
@@ -1327,6 +1330,7 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
     }
     const int head = g * G + mt * 16 + rr;
     if (p.num_splits == 1) {
+      if (p.sinks && mx != -INFINITY) den += fast_exp2(p.sinks[head] * 1.4426950408889634f - mx);
       p.out[(long long)tok * p.nq * D + (long long)head * D + d] = (bf16_t)(num / den);
     } else {
       const long long slot = ((long long)w * p.nq + head) * p.num_splits + split;
@@ -1376,6 +1380,7 @@ __global__ void attn_decode_merge_kernel(AttnArgs p) {
       den += live ? v[i].y * f : 0.f;
     }
   }
+  if (p.sinks && mx != -INFINITY) den += fast_exp2(p.sinks[head] * 1.4426950408889634f - mx);      // once, after all splits
   if (threadIdx.x < D) p.out[(long long)tok * p.nq * D + (long long)head * D + d] = (bf16_t)(num / den);
 }
 
@@ -1397,9 +1402,10 @@ extern "C" int jv_attn_prefill(void* out, const void* q, long long q_row_stride,
                                const void* v_pages, const int* block_tables, int table_stride,
                                const int* cu_seqlens, const int* context_lens, const int* work,
                                int n_work, int page_size, int nq, int nkv, float scale, int window,
-                               void* stream) {
+                               const float* sinks, void* stream) {
   if (n_work <= 0) return 0;
   AttnArgs a{};
+  a.sinks = sinks;
   a.out = (bf16_t*)out; a.q = (const bf16_t*)q; a.q_row_stride = q_row_stride;
   a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
   a.block_tables = block_tables; a.table_stride = table_stride;
@@ -1431,9 +1437,10 @@ extern "C" int jv_attn_decode(void* out, const void* q, long long q_row_stride, 
                               const void* v_pages, const int* block_tables, int table_stride,
                               const int* cu_seqlens, const int* context_lens, const int* work,
                               int n_work, int page_size, int nq, int nkv, float scale, int window,
-                              int num_splits, float* scratch, void* stream) {
+                              int num_splits, float* scratch, const float* sinks, void* stream) {
   if (n_work <= 0) return 0;
   AttnArgs a{};
+  a.sinks = sinks;
   a.out = (bf16_t*)out; a.q = (const bf16_t*)q; a.q_row_stride = q_row_stride;
   a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
   a.block_tables = block_tables; a.table_stride = table_stride;

@@ -199,7 +199,7 @@ def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
     _check(fn(_ptr(rows), _ptr(bias), c_longlong(rows.shape[0]), c_int(rows.shape[1]), _stream()), "add_bias")
 
 
-PLAIN_ACTIVATIONS = {None: 0, "silu": 1, "gelu_tanh": 2, "gelu": 3}     # ids of act in y = act(x + bias); "gelu" is the erf form
+PLAIN_ACTIVATIONS = {None: 0, "silu": 1, "gelu_tanh": 2, "gelu": 3, "tanh": 4}     # ids of act in y = act(x + bias); "gelu" is the erf form
 
 
 def bias_act(y: torch.Tensor, bias, activation) -> None:
@@ -232,22 +232,23 @@ def scaled_sum(out: torch.Tensor, y, scale: float) -> None:
               c_longlong(0 if parts is None else parts.stride(0)), c_longlong(out.numel()), c_float(scale), _stream()), "scaled_sum")
 
 
-def embedding_pair(h: torch.Tensor, table: torch.Tensor, pair: torch.Tensor, ids: torch.Tensor, prev: torch.Tensor,
-                   buckets: int, mul_prev: int, mul_cur: int) -> None:
-    """h[t] = float(table[ids[t]]) + float(pair[r]) with r = (prev[t] * mul_prev + ids[t] * mul_cur) mod buckets, or
-    r = buckets (the last row of ``pair``) where prev[t] < 0: a sequence's first token."""
+def embedding_pair(h: torch.Tensor, table: torch.Tensor, pair, ids: torch.Tensor, prev: torch.Tensor,
+                   buckets: int, mul_prev: int, mul_cur: int, scale: float = 1.0) -> None:
+    """h[t] = scale * float(table[ids[t]]) + float(pair[r]) with r = (prev[t] * mul_prev + ids[t] * mul_cur) mod buckets,
+    or r = buckets (the last row of ``pair``) where prev[t] < 0: a sequence's first token.  ``pair`` None: the scaled
+    row alone."""
     _dev(h, table, pair, ids, prev)
     n, hidden = h.shape
     _f32(h, "h")
     _i32(ids, "ids", n)
     _i32(prev, "prev", n)
     _need(table.dim() == 2 and table.shape[1] == hidden and table.is_contiguous(), "table width differs from h")
-    _need(pair.shape == (buckets + 1, hidden) and pair.dtype == table.dtype and pair.is_contiguous(),
+    _need(pair is None or (pair.shape == (buckets + 1, hidden) and pair.dtype == table.dtype and pair.is_contiguous()),
           "the pair table must be [buckets + 1, hidden] of the table's type")
     _need(buckets > 0 and 0 <= mul_prev < 2 ** 31 and 0 <= mul_cur < 2 ** 31, "buckets must be positive, the multipliers below 2^31")
     fn = getattr(library.core(), f"jv_embedding_pair_{_suffix(table.dtype)}")
     _check(fn(_ptr(h), _ptr(table), _ptr(pair), _ptr(ids), _ptr(prev), c_int(n), c_int(hidden), c_int(table.shape[0]),
-              c_longlong(buckets), c_longlong(mul_prev), c_longlong(mul_cur), _stream()), "embedding_pair")
+              c_longlong(buckets), c_longlong(mul_prev), c_longlong(mul_cur), c_float(scale), _stream()), "embedding_pair")
 
 
 def add_outputs(h: torch.Tensor, a, b=None, out_dtype=None):
@@ -427,19 +428,32 @@ def padded_head_dim(dk: int, dv: int) -> int:
 
 def attn_prepare_wide(qkv, bias, q_weight, k_weight, eps: float, cos_sin, rot_dims: int, slot_mapping, k_pages, v_pages,
                       page_size: int, nq: int, nkv: int, dk: int, dv: int, dp: int, v_scale: float = 1.0,
-                      norm_per_head: bool = False) -> torch.Tensor:
+                      norm_per_head: bool = False, values_are_keys: bool = False, positions=None,
+                      q_temperature: "tuple | None" = None) -> torch.Tensor:
     """Attention input whose key and value sizes differ, whose q/k norm spans the whole projection, or whose rows
     carry more than q, k and v.  ``qkv`` rows
     begin with [q: nq * dk | k: nkv * dk | v: nkv * dv] (further columns are left alone); ``bias`` (float32, that width) is added first; with
     ``q_weight`` [nq * dk] and ``k_weight`` [nkv * dk] q and k are RMS-normed over all their columns at once (with
     ``norm_per_head``: every head on its own, with weights [dk] shared by the heads); the
     first ``rot_dims`` elements of every q and k head turn by ``cos_sin`` (``rope_table``); v is multiplied by
-    ``v_scale``.  Returns q as [n, nq * dp] with every head padded with zeros to ``dp``; keys go to
+    ``v_scale``.  ``values_are_keys``: the rows hold [q | k] only and the values are the k columns as projected (before
+    bias-free norm and rotation; needs dv == dk and no whole-projection norm).  ``q_temperature`` (coef, every) with
+    ``positions`` (int32 [n]): q at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).  Returns q as [n, nq * dp] with every head padded with zeros to ``dp``; keys go to
     [pages, nkv, page_size, dp], values to [pages, nkv, dp, page_size] (their pad is never written)."""
     _dev(qkv, bias, q_weight, k_weight, cos_sin, slot_mapping, k_pages, v_pages)
     n, ld = qkv.shape
-    width = (nq + nkv) * dk + nkv * dv
+    v_off = nq * dk if values_are_keys else (nq + nkv) * dk
+    width = v_off + nkv * dv
+    _need(not values_are_keys or (dv == dk and (q_weight is None or norm_per_head)),
+          "values that are the keys have the keys' size, and the norm is per head or none")
     _need(qkv.dim() == 2 and ld >= width and qkv.is_contiguous(), "qkv rows must begin with nq * dk + nkv * dk + nkv * dv columns")
+    coef, every = (0.0, 1)
+    if q_temperature is not None:
+        coef, every = float(q_temperature[0]), int(q_temperature[1])
+        _need(every > 0 and positions is not None and (q_weight is None or norm_per_head),
+              "a query temperature needs positions, a positive period and a per-head norm or none")
+        _dev(positions)
+        _i32(positions, "positions", n)
     _need(dp >= max(dk, dv), "the padded head size must hold keys and values")
     if bias is not None:
         _f32(bias, "bias", width)
@@ -458,17 +472,21 @@ def attn_prepare_wide(qkv, bias, q_weight, k_weight, eps: float, cos_sin, rot_di
     _check(fn(_ptr(q), _ptr(qkv), c_longlong(ld), _ptr(bias), _ptr(q_weight), _ptr(k_weight), c_float(eps),
               _ptr(cos_sin if rot_dims else None), c_int(rot_dims), _ptr(slot_mapping if k_pages is not None else None),
               _ptr(k_pages), _ptr(v_pages), c_int(page_size), c_int(n), c_int(nq), c_int(nkv), c_int(dk), c_int(dv),
-              c_int(dp), c_float(v_scale), c_int(1 if norm_per_head else 0), _stream()), "attn_prepare_wide")
+              c_int(dp), c_float(v_scale), c_int(1 if norm_per_head else 0), c_longlong(v_off),
+              _ptr(positions if q_temperature is not None else None), c_float(coef), c_int(every), _stream()), "attn_prepare_wide")
     return q
 
 
 # --------------------------------------------------------------------------- attention
 def paged_attention_generic(out, q, q_row_stride, k_pages, v_pages, block_tables, token_req, positions,
-                            nq, nkv, head_dim, scale, window=0) -> None:
+                            nq, nkv, head_dim, scale, window=0, sinks=None) -> None:
     """Causal attention of every token over its request's pages (generic float-math kernel).
 
-    ``q`` is any tensor whose row t holds the q heads at [t * q_row_stride + h * D]."""
-    _dev(out, q, k_pages, v_pages, block_tables, token_req, positions)
+    ``q`` is any tensor whose row t holds the q heads at [t * q_row_stride + h * D].  ``sinks`` (float32 [nq]):
+    exp(sinks[h]) joins every row's softmax denominator (a term without key and value, not scaled)."""
+    _dev(out, q, k_pages, v_pages, block_tables, token_req, positions, sinks)
+    if sinks is not None:
+        _f32(sinks, "sinks", nq)
     n = out.shape[0]
     _need(out.shape == (n, nq * head_dim) and out.dtype == q.dtype, "out must be [tokens, nq * D] of q's type")
     _need(q.numel() >= (n - 1) * q_row_stride + nq * head_dim if n else True, "q is too small for its stride")
@@ -484,7 +502,7 @@ def paged_attention_generic(out, q, q_row_stride, k_pages, v_pages, block_tables
     _check(
         fn(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages), _ptr(block_tables),
            c_int(block_tables.shape[1]), _ptr(token_req), _ptr(positions), c_int(page_size), c_int(n),
-           c_int(nq), c_int(nkv), c_int(head_dim), c_float(scale), c_int(window or 0), _stream()),
+           c_int(nq), c_int(nkv), c_int(head_dim), c_float(scale), c_int(window or 0), _ptr(sinks), _stream()),
         "paged_attention_generic",
     )
 
@@ -855,12 +873,20 @@ def _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlen
     return page_size
 
 
+def _sinks_ok(sinks, nq: int) -> None:
+    if sinks is not None:
+        _dev(sinks)
+        _f32(sinks, "sinks", nq)
+
+
 def attn_prefill_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, n_work,
-                      nq, nkv, head_dim, scale, window=0) -> None:
+                      nq, nkv, head_dim, scale, window=0, sinks=None) -> None:
     """Causal attention of prompt portions.  ``work`` is int32 [n_work, 3]: (request index, first row
     of a group, first row of a second group of the same request or -1), see ``attn_prefill_geometry``;
     every row of every request must be in exactly one group.  Pairing a group that sees many keys with
-    one that sees few gives all blocks the same amount of work."""
+    one that sees few gives all blocks the same amount of work.  ``sinks`` (float32 [nq]): exp(sinks[h]) joins every
+    row's softmax denominator (a term without key and value, not scaled)."""
+    _sinks_ok(sinks, nq)
     page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
                              nq, nkv, head_dim)
     _need(work.numel() >= 3 * n_work, "work list shorter than n_work")
@@ -869,7 +895,7 @@ def attn_prefill_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_s
         lib.jv_attn_prefill(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages),
                             _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens),
                             _ptr(work), c_int(n_work), c_int(page_size), c_int(nq), c_int(nkv), c_float(scale),
-                            c_int(window or 0), _stream()),
+                            c_int(window or 0), _ptr(sinks), _stream()),
         "attn_prefill_mfma",
     )
 
@@ -894,12 +920,14 @@ def attn_decode_scratch_floats(n_work: int, nq: int, num_splits: int, head_dim: 
 
 
 def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, n_work,
-                     nq, nkv, head_dim, scale, window=0, num_splits=1, scratch=None) -> None:
+                     nq, nkv, head_dim, scale, window=0, num_splits=1, scratch=None, sinks=None) -> None:
     """Attention of single decoded tokens.  ``work`` is int32 [n_work]: indices of the requests
     (each with exactly one token in this step); None: the step holds decoded tokens only, request
     r = 0 .. n_work-1 has its token in row r (the kernel then has nothing to look up before its
     loads start).  With ``num_splits`` > 1 a request's keys are shared out to that many blocks and
-    ``scratch`` (float32, ``attn_decode_scratch_floats`` entries) holds their partial results."""
+    ``scratch`` (float32, ``attn_decode_scratch_floats`` entries) holds their partial results.  ``sinks``: as for
+    ``attn_prefill_mfma`` (counted once, after the splits are merged)."""
+    _sinks_ok(sinks, nq)
     page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
                              nq, nkv, head_dim)
     if work is None:
@@ -920,7 +948,7 @@ def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_se
                            _ptr(cu_seqlens if work is not None else None), _ptr(context_lens),
                            _ptr(work), c_int(n_work), c_int(page_size), c_int(nq), c_int(nkv), c_float(scale),
                            c_int(window or 0), c_int(num_splits), _ptr(scratch if num_splits > 1 else None),
-                           _stream()),
+                           _ptr(sinks), _stream()),
         "attn_decode_mfma",
     )
 
@@ -955,9 +983,10 @@ class PendingNorm:
     joins the residual stream: what a layer arrangement that norms the output of its sublayers hands
     to the next norm, which does both in one pass (``postnorm_add_rmsnorm``)."""
 
-    def __init__(self, y, parts, weight: torch.Tensor, eps: float, bias=None):
+    def __init__(self, y, parts, weight, eps: float, bias=None, scale: float = 1.0):
         self.y, self.parts, self.weight, self.eps = y, parts, weight, float(eps)
         self.bias = bias          # float [hidden] or None: a bias of the sublayer's last product, still to be added
+        self.scale = float(scale)  # with ``weight`` None: no norm at all, the sum joins the stream times this constant
 
 
 class BiasedOutput:
@@ -994,17 +1023,27 @@ def pending_norm(out, weight: torch.Tensor, eps: float) -> "PendingNorm":
     return PendingNorm(*split_sublayer_output(out), weight, eps)
 
 
+def pending_scale(out, scale: float) -> "PendingNorm":
+    """A sublayer's output that joins the residual stream multiplied by a constant (no norm of its own): the next
+    norm's kernel adds ``scale`` times the output (rows plus float partial results) and norms the stream in one pass."""
+    if isinstance(out, BiasedOutput):
+        out = out.settled()
+    return PendingNorm(*split_sublayer_output(out), None, 0.0, None, scale)
+
+
 def postnorm_add_rmsnorm(h, y, parts, post_weight, eps: float, weight=None, out=None, rows=None,
-                         out_eps: float | None = None, bias=None) -> None:
+                         out_eps: float | None = None, bias=None, plain_scale: float = 1.0) -> None:
     """h += norm(y + parts[0] + parts[1] + ... (+ bias); post_weight) in the float residual stream, then, with
     ``out``, out = norm(h; weight) (with ``out_eps``, default ``eps``) in the activation type, or h itself in that type where
     ``weight`` is None (a reader that takes the stream as it is).  With ``rows`` (int32 indices) only those
-    rows are computed and h is left alone.  y is [rows of h, hidden] in the activation type or None,
+    rows are computed and h is left alone.  ``post_weight`` None: the sublayer's output joins the stream under a constant
+    only, h += plain_scale * (y + parts ...).  y is [rows of h, hidden] in the activation type or None,
     parts a float32 stack [P, rows of h, hidden] or None (any P)."""
     _dev(h, y, parts, post_weight, weight, out, rows, bias)
     _f32(h, "h")
     n, hidden = h.shape
-    _f32(post_weight, "post_weight", hidden)
+    if post_weight is not None:
+        _f32(post_weight, "post_weight", hidden)
     if bias is not None:       # added to the sublayer's output before its norm
         _f32(bias, "bias", hidden)
     _need(y is not None or parts is not None, "nothing to add")
@@ -1031,7 +1070,7 @@ def postnorm_add_rmsnorm(h, y, parts, post_weight, eps: float, weight=None, out=
     fn = getattr(library.core(), f"jv_postnorm_add_rmsnorm_{_suffix(kind)}")
     _check(fn(_ptr(h), _ptr(y), _ptr(parts), c_int(0 if parts is None else parts.shape[0]),
               c_longlong(0 if parts is None else parts.stride(0)), _ptr(bias), _ptr(post_weight), _ptr(weight), _ptr(out),
-              _ptr(rows), c_int(n_out), c_int(hidden), c_float(eps), c_float(eps if out_eps is None else out_eps), _stream()),
+              _ptr(rows), c_int(n_out), c_int(hidden), c_float(eps), c_float(eps if out_eps is None else out_eps), c_float(plain_scale), _stream()),
            "postnorm_add_rmsnorm")
 
 
@@ -1064,14 +1103,18 @@ def rope_table_amp(positions: torch.Tensor, inv_freq: torch.Tensor, amplitude: f
 
 
 def latent_prepare(proj, q_rank: int, rank: int, rot: int, rot_dims: int, q_weight, kv_weight, eps: float, cos_sin,
-                   slot_mapping, k_pages, v_pages, page_size: int) -> torch.Tensor:
+                   slot_mapping, k_pages, v_pages, page_size: int, kv_off: "int | None" = None,
+                   interleaved: bool = False):
     """From rows ``proj`` = [q latent | kv latent | key part to rotate | ...]: returns the normed q latent
-    [n, q_rank]; stores [normed kv latent | rotated key part] of every token with a slot (>= 0) into its key
+    [n, q_rank] (None for ``q_rank`` 0: queries that are projected directly; the kv latent then begins at column
+    ``kv_off``, default ``q_rank``); ``interleaved``: the pairs (2i, 2i + 1) turn instead of (i, i + rot_dims / 2); stores [normed kv latent | rotated key part] of every token with a slot (>= 0) into its key
     page [pages, 1, page_size, rank + rot] and transposed value page [pages, 1, rank + rot, page_size]."""
     _dev(proj, q_weight, kv_weight, cos_sin, slot_mapping, k_pages, v_pages)
     n, ld = proj.shape
-    _need(ld >= q_rank + rank + rot, "proj rows are too short")
-    _f32(q_weight, "q_weight", q_rank)
+    kv_off = q_rank if kv_off is None else int(kv_off)
+    _need(q_rank >= 0 and kv_off >= q_rank and ld >= kv_off + rank + rot, "proj rows are too short")
+    if q_rank:
+        _f32(q_weight, "q_weight", q_rank)
     _f32(kv_weight, "kv_weight", rank)
     _need(rot_dims % 2 == 0 and 0 <= rot_dims <= rot, "the rotated size must be even and at most the key part")
     if rot_dims:
@@ -1079,31 +1122,35 @@ def latent_prepare(proj, q_rank: int, rank: int, rot: int, rot_dims: int, q_weig
     if k_pages is not None:
         _i32(slot_mapping, "slot_mapping", n)
         _check_pages(k_pages, v_pages, proj.dtype, 1, page_size, rank + rot)
-    cq = torch.empty((n, q_rank), dtype=proj.dtype, device=proj.device)
+    cq = torch.empty((n, q_rank), dtype=proj.dtype, device=proj.device) if q_rank else None
     fn = getattr(library.core(), f"jv_latent_prepare_{_suffix(proj.dtype)}")
-    _check(fn(_ptr(proj), c_longlong(ld), c_int(n), c_int(q_rank), c_int(rank), c_int(rot), c_int(rot_dims),
-              _ptr(q_weight), _ptr(kv_weight), c_float(eps), _ptr(cos_sin),
+    _check(fn(_ptr(proj), c_longlong(ld), c_int(n), c_int(q_rank), c_longlong(kv_off), c_int(rank), c_int(rot), c_int(rot_dims),
+              c_int(1 if interleaved else 0), _ptr(q_weight if q_rank else None), _ptr(kv_weight), c_float(eps),
+              _ptr(cos_sin if rot_dims else None),
               _ptr(slot_mapping if k_pages is not None else None), _ptr(cq), _ptr(k_pages), _ptr(v_pages),
               c_int(page_size), _stream()), "latent_prepare")
     return cq
 
 
-def latent_query_rope(q, qe, heads: int, dim: int, rot: int, rot_dims: int, rank: int, cos_sin) -> None:
-    """qe[t, h, rank:] = rotate(q[t, h, dim:]) for q [n, heads * (dim + rot)], qe [n, heads * (rank + rot)]."""
+def latent_query_rope(q, qe, heads: int, dim: int, rot: int, rot_dims: int, rank: int, cos_sin,
+                      interleaved: bool = False) -> None:
+    """qe[t, h, rank:] = rotate(q[t, h, dim:]) for q rows that begin with heads * (dim + rot) columns (further columns
+    are left alone), qe [n, heads * (rank + rot)]; ``interleaved``: the pairs (2i, 2i + 1) turn."""
     _dev(q, qe, cos_sin)
     n = q.shape[0]
-    _need(q.shape == (n, heads * (dim + rot)) and qe.shape == (n, heads * (rank + rot)) and q.dtype == qe.dtype,
-          "q must be [n, heads * (dim + rot)], qe [n, heads * (rank + rot)] of one type")
+    _need(q.dim() == 2 and q.shape[1] >= heads * (dim + rot) and qe.shape == (n, heads * (rank + rot)) and q.dtype == qe.dtype,
+          "q rows must begin with heads * (dim + rot) columns, qe be [n, heads * (rank + rot)] of one type")
     if rot_dims:
         _f32(cos_sin, "cos_sin", n * rot_dims)
     fn = getattr(library.core(), f"jv_latent_query_rope_{_suffix(q.dtype)}")
-    _check(fn(_ptr(q), _ptr(qe), c_int(n), c_int(heads), c_int(dim), c_int(rot), c_int(rot_dims), c_int(rank),
-              _ptr(cos_sin), _stream()), "latent_query_rope")
+    _check(fn(_ptr(q), c_longlong(q.shape[1]), _ptr(qe), c_int(n), c_int(heads), c_int(dim), c_int(rot), c_int(rot_dims),
+              c_int(rank), _ptr(cos_sin if rot_dims else None), c_int(1 if interleaved else 0), _stream()), "latent_query_rope")
 
 
 def head_linear(y, y_head_stride: int, x, x_head_stride: int, w, gate=None, matrix_cores: "bool | None" = None) -> None:
     """One matrix per head: y[t, h * ys : h * ys + N] = w[h] @ x[t, h * xs : h * xs + K], w [heads, N, K];
-    with ``gate`` (a [n, heads * N] view with unit column stride) the result is multiplied by sigmoid(gate).
+    with ``gate`` (a [n, heads * N] view with unit column stride) the result is multiplied by sigmoid(gate); a gate
+    view [n, heads] holds one number per head, for all of the head's outputs.
     x and y are row-major matrices of the activation type; float accumulation.  bfloat16 with K, the row
     stride and the head stride of x multiples of 8 runs on the matrix cores (``matrix_cores`` False: the
     float-FMA kernels all the same)."""
@@ -1115,8 +1162,8 @@ def head_linear(y, y_head_stride: int, x, x_head_stride: int, w, gate=None, matr
     _need((heads - 1) * x_head_stride + K <= x.shape[1] and (heads - 1) * y_head_stride + N <= y.shape[1],
           "heads do not fit the rows")
     if gate is not None:
-        _need(gate.is_cuda and gate.dtype == x.dtype and gate.shape == (n, heads * N) and gate.stride(1) == 1,
-              "gate must be a [n, heads * N] view with unit column stride")
+        _need(gate.is_cuda and gate.dtype == x.dtype and gate.shape in ((n, heads * N), (n, heads)) and gate.stride(1) == 1,
+              "gate must be a [n, heads * N] or [n, heads] view with unit column stride")
     possible = (x.dtype == torch.bfloat16 and K >= 8 and K % 8 == 0 and x.shape[1] % 8 == 0 and x_head_stride % 8 == 0
                 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
     _need(not matrix_cores or possible, "the matrix-core kernel takes bfloat16 and sizes and strides that are multiples of 8")
@@ -1124,7 +1171,8 @@ def head_linear(y, y_head_stride: int, x, x_head_stride: int, w, gate=None, matr
     fn = getattr(library.core(), name)
     _check(fn(_ptr(y), c_longlong(y.shape[1]), c_int(y_head_stride), _ptr(x), c_longlong(x.shape[1]),
               c_int(x_head_stride), _ptr(w), c_int(n), c_int(N), c_int(K), c_int(heads), _ptr(gate),
-              c_longlong(0 if gate is None else gate.stride(0)), _stream()), "head_linear")
+              c_longlong(0 if gate is None else gate.stride(0)),
+              c_int(N if gate is None or gate.shape[1] == heads * N else 1), _stream()), "head_linear")
 
 
 # --------------------------------------------------------------------------- linear attention with decay
@@ -1357,6 +1405,54 @@ def recurrence_steps(q, k, v, decay, state, slot_ids, cu_seqlens, heads: int, qk
     return out
 
 
+def token_shift_mix(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, slot_ids, cu_seqlens, token_req) -> torch.Tensor:
+    """Blends of every row with the row before it in its request: returns [S, n, hidden] of x's type with
+    out[s, t] = x[t] + (x[t-1] - x[t]) * mu[s] (float arithmetic); ``mu`` float32 [S, hidden].  The row before a
+    request's first row of the step is the request's row of ``state`` (float32 [slots + 1, hidden], zeros for a
+    request that starts), which then takes the request's last row of the step."""
+    _dev(x, mu, state, slot_ids, cu_seqlens, token_req)
+    n, hidden = x.shape
+    _f32(mu, "mu")
+    _need(mu.dim() == 2 and mu.shape[1] == hidden, "mu must be [S, hidden]")
+    _f32(state, "state")
+    _need(state.dim() == 2 and state.shape[1] == hidden, "the state must be [slots + 1, hidden]")
+    _i32(slot_ids, "slot_ids")
+    _i32(cu_seqlens, "cu_seqlens", slot_ids.numel() + 1)
+    _i32(token_req, "token_req", n)
+    out = torch.empty((mu.shape[0], n, hidden), dtype=x.dtype, device=x.device)
+    fn = getattr(library.core(), f"jv_token_shift_mix_{_suffix(x.dtype)}")
+    _check(fn(_ptr(out), _ptr(x), _ptr(mu), c_int(mu.shape[0]), _ptr(state), _ptr(slot_ids), _ptr(cu_seqlens), _ptr(token_req),
+              c_longlong(n), c_int(hidden), _stream()), "token_shift_mix")
+    return out
+
+
+WKV_MAX_DIM = 8192      # 32 rows of a column in each of a block's 256 threads
+
+
+def wkv_steps(r, k, v, rate, w0, bonus, state, slot_ids, cu_seqlens, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """The recurrence with a decay per key channel and a bonus for the current token, per head with S the request's
+    float state [dim, vdim]:  w = exp(-exp(rate + w0));  o = S^T r + (sum_d r[d] bonus[d] k[d]) v;  S <- diag(w) S + k v^T.
+    r, k, rate [n, heads * dim] and v [n, heads * vdim] are views (unit column stride) of the activation type; w0 and
+    bonus float32 [heads * dim]; ``state`` float32 [slots + 1, heads, dim, vdim].  Returns float32 [n, heads * vdim]."""
+    _dev(w0, bonus, state, slot_ids, cu_seqlens)
+    n = r.shape[0]
+    for name, t, width in (("r", r, heads * dim), ("k", k, heads * dim), ("rate", rate, heads * dim), ("v", v, heads * vdim)):
+        _need(t.is_cuda and t.dtype == r.dtype and t.shape == (n, width) and (n == 0 or t.stride(1) == 1),
+              f"{name} must be a [n, {width}] view with unit column stride of one type")
+    _f32(w0, "w0", heads * dim)
+    _f32(bonus, "bonus", heads * dim)
+    _f32(state, "state")
+    _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, dim, vdim), "the state must be [slots + 1, heads, dim, vdim]")
+    _i32(slot_ids, "slot_ids")
+    _i32(cu_seqlens, "cu_seqlens", slot_ids.numel() + 1)
+    out = torch.empty((n, heads * vdim), dtype=torch.float32, device=r.device)
+    fn = getattr(library.core(), f"jv_wkv_steps_{_suffix(r.dtype)}")
+    _check(fn(_ptr(out), _ptr(r), c_longlong(r.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
+              _ptr(rate), c_longlong(rate.stride(0)), _ptr(w0), _ptr(bonus), _ptr(state), _ptr(slot_ids), _ptr(cu_seqlens),
+              c_int(slot_ids.numel()), c_int(heads), c_int(dim), c_int(vdim), _stream()), "wkv_steps")
+    return out
+
+
 RECURRENCE_CHUNK_MIN_TOKENS = 8     # from this many tokens of a request on, the kernels by chunks
 
 
@@ -1463,15 +1559,18 @@ class MoePlan:
         self.tile_rows = tile_rows
 
 
-ROUTER_SCORES = {"sigmoid": 0, "softmax_chosen": 1}      # the kernels' ids of how a chosen logit becomes a weight
+ROUTER_SCORES = {"sigmoid": 0, "softmax_chosen": 1, "sigmoid_normed": 2}      # the kernels' ids of how a chosen logit becomes a weight
 
 
 def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, logits_out=None,
-              tile_rows: "int | None" = None, bias=None, score: str = "sigmoid") -> MoePlan:
+              tile_rows: "int | None" = None, bias=None, score: str = "sigmoid", correction=None,
+              weight_scale: float = 1.0) -> MoePlan:
     """Chooses for every token the ``top`` experts with the largest router logits (the lowest index among equal
     logits) and orders the n * top entries by expert, all on the device.  ``bias`` (float32 [experts]) is added
     to the logits before the choice; ``score``: a chosen expert's weight is "sigmoid" of its logit, or
-    "softmax_chosen": the softmax over the token's chosen logits alone.
+    "softmax_chosen": the softmax over the token's chosen logits alone, or "sigmoid_normed": the experts with the
+    largest sigmoid(logit) + ``correction`` (float32 [experts] or None) are chosen, and a chosen expert's weight is its
+    sigmoid(logit) (without the correction) over the sum of the chosen ones' (+ 1e-20), times ``weight_scale``.
     Either float ``logits`` [n, experts] are given, or rows ``x`` [n, hidden] and the router matrix
     ``w_router`` [experts, hidden] of one type: then the logits are made here, in float (``logits_out``,
     float32 [n, experts], receives them if given): in the same launch as the choice (float32, odd sizes), or
@@ -1509,6 +1608,11 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
     if bias is not None:
         _dev(bias)
         _f32(bias, "bias", experts)
+    _need(score == "sigmoid_normed" or (correction is None and weight_scale == 1.0),
+          "a correction of the choice and a constant on the weights belong to the score 'sigmoid_normed'")
+    if correction is not None:
+        _dev(correction)
+        _f32(correction, "correction", experts)
     entries = n * top
     tile_rows = tile_rows or moe_tile_rows()
     _need(tile_rows in (64, 128), "tiles have 64 or 128 rows")
@@ -1523,14 +1627,26 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
     lib = library.core()
     if logits is not None:
         _check(lib.jv_moe_route(_ptr(logits), _ptr(bias), c_int(n), c_int(experts), c_int(top), c_int(ROUTER_SCORES[score]),
-                                _ptr(ids), _ptr(weights), _stream()), "moe_route")
+                                _ptr(ids), _ptr(weights), _ptr(correction), c_float(weight_scale), _stream()), "moe_route")
     else:
         _check(getattr(lib, f"jv_moe_router_{_suffix(x.dtype)}")(
             _ptr(x), _ptr(w_router), _ptr(bias), c_int(n), c_int(hidden), c_int(experts), c_int(top),
-            c_int(ROUTER_SCORES[score]), _ptr(ids), _ptr(weights), _ptr(logits_out), _stream()), "moe_router")
+            c_int(ROUTER_SCORES[score]), _ptr(ids), _ptr(weights), _ptr(logits_out), _ptr(correction),
+            c_float(weight_scale), _stream()), "moe_router")
     _check(lib.jv_moe_group(_ptr(ids), c_int(entries), c_int(experts), c_int(tile_rows), _ptr(meta), _ptr(offsets), _ptr(tile_expert),
                             _ptr(tile_row0), _ptr(order), _ptr(rank), _stream()), "moe_group")
     return MoePlan(ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top, tile_rows)
+
+
+def row_gate(out: torch.Tensor, y: torch.Tensor, gate: torch.Tensor) -> None:
+    """out[t] = float(y[t]) * sigmoid(gate[t]): rows ``y`` [n, hidden] of the activation type under one gate per row
+    (``gate`` a [n, 1] view of the same type, any row stride), into float32 ``out`` [n, hidden]."""
+    _dev(out, y)
+    n, hidden = y.shape
+    _need(out.dtype == torch.float32 and out.shape == y.shape, "out must be float32 of y's shape")
+    _need(gate.is_cuda and gate.dtype == y.dtype and gate.shape == (n, 1), "gate must be a [n, 1] view of y's type")
+    fn = getattr(library.core(), f"jv_row_gate_{_suffix(y.dtype)}")
+    _check(fn(_ptr(out), _ptr(y), _ptr(gate), c_longlong(gate.stride(0)), c_longlong(n), c_int(hidden), _stream()), "row_gate")
 
 
 def moe_matrix_cores_possible(dtype, hidden: int, ff: int) -> bool:

@@ -25,12 +25,15 @@ class GroupedQueryAttention:
                  qk_norm_eps: Optional[float] = None, position: Optional[PartSpec] = None,
                  window: Optional[int] = None, scale: Optional[float] = None, qkv_bias: bool = False,
                  o_bias: bool = False, v_head_dim: Optional[int] = None, qk_norm: str = "head", v_scale: float = 1.0,
-                 output_gate: bool = False):
+                 output_gate: bool = False, values_are_keys: bool = False, q_temperature: Optional[tuple] = None):
         """``v_head_dim``: a value size that differs from the key size; ``qk_norm`` "whole": the q/k norm spans all
         of q's (and all of k's) columns at once, with weights of that size, instead of every head on its own;
         ``v_scale``: a constant on the values (and so on the mixer's result before its output projection);
         ``output_gate``: the concatenated heads are multiplied by sigmoid(W_g x) before the output projection (W_g is
-        one more block of rows of the fused input projection).  Any of the four takes the ``wide`` path: heads cached
+        one more block of rows of the fused input projection);
+        ``values_are_keys``: there is no value projection, the values are the keys as projected (before their norm and
+        rotation); ``q_temperature`` (coef, every): the query at position p is multiplied by
+        1 + coef * ln(floor((p + 1) / every) + 1), after its norm.  Any of these takes the ``wide`` path: heads cached
         under one padded size (``K.padded_head_dim``), prepared by ``K.attn_prepare_wide``, read by the same paged
         attention kernels."""
         if num_heads % num_kv_heads:
@@ -42,7 +45,13 @@ class GroupedQueryAttention:
         self.dv = int(v_head_dim) if v_head_dim else self.dk
         self.qk_norm, self.v_scale = qk_norm, float(v_scale)
         self.output_gate = bool(output_gate)
-        self.wide = (self.dv != self.dk or (qk_norm == "whole" and qk_norm_eps is not None) or self.v_scale != 1.0
+        self.values_are_keys = bool(values_are_keys)
+        self.q_temperature = (float(q_temperature[0]), int(q_temperature[1])) if q_temperature else None
+        if self.q_temperature is not None and self.q_temperature[1] <= 0:
+            raise ValueError("the period of a query temperature must be positive")
+        if self.values_are_keys and (self.dv != self.dk or qkv_bias or (qk_norm == "whole" and qk_norm_eps is not None)):
+            raise ValueError("values that are the keys: one head size, no input bias, a per-head q/k norm or none")
+        self.wide = (self.values_are_keys or self.q_temperature is not None or self.dv != self.dk or (qk_norm == "whole" and qk_norm_eps is not None) or self.v_scale != 1.0
                      or self.output_gate)
         # what the paged attention kernels see
         self.d = K.padded_head_dim(self.dk, self.dv) if self.wide else self.dk
@@ -73,6 +82,8 @@ class GroupedQueryAttention:
             "v_proj.weight": TensorSpec((self.nkv * self.dv, self.hidden_size)),
             "o_proj.weight": TensorSpec((self.hidden_size, self.nq * self.dv)),
         }
+        if self.values_are_keys:
+            del t["v_proj.weight"]
         if self.qk_norm_eps is not None:
             whole = self.qk_norm == "whole"
             t["q_norm.weight"] = TensorSpec((self.nq * self.dk if whole else self.dk,), role="vector", init="norm")
@@ -96,11 +107,13 @@ class GroupedQueryAttention:
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
         self.dtype = dtype
         # one product for everything that reads the input: q, k, v and, behind them, the gate's rows
-        blocks = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+        blocks = [tensors["q_proj.weight"], tensors["k_proj.weight"]]
+        if not self.values_are_keys:
+            blocks.append(tensors["v_proj.weight"])
         if self.output_gate:
             blocks.append(tensors["gate.weight"])
         self.w_qkv = torch.cat(blocks, dim=0).contiguous()
-        self.qkv_width = self.nq * self.dk + self.nkv * (self.dk + self.dv)
+        self.qkv_width = self.nq * self.dk + self.nkv * (self.dk + (0 if self.values_are_keys else self.dv))
         self.w_o = tensors["o_proj.weight"]
         if self.wide and self.d != self.dv:
             # the attention's result has heads of the padded size (zeros behind the values): zero columns there
@@ -169,7 +182,8 @@ class GroupedQueryAttention:
             qkv, self.b_qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos_sin, rotary_dim,
             ctx.slot_mappings[mem.group] if writes else None, mem.pages["k"] if writes else None,
             mem.pages["v"] if writes else None, ctx.page_size, self.nq, self.nkv, self.dk, self.dv, self.d, self.v_scale,
-            norm_per_head=self.qk_norm == "head")
+            norm_per_head=self.qk_norm == "head", values_are_keys=self.values_are_keys,
+            positions=ctx.positions if self.q_temperature is not None else None, q_temperature=self.q_temperature)
         out = torch.empty((qkv.shape[0], self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
         from . import attention_backend
 

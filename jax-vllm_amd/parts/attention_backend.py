@@ -146,10 +146,11 @@ def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> Mfm
 def run(att, out, qkv, ctx, mem) -> None:
     # q heads of a row sit at the front of the fused q/k/v projection, unless the mixer says where else
     q_row_stride = getattr(att, "q_row_stride", None) or (att.nq + 2 * att.nkv) * att.d
+    sinks = getattr(att, "sinks", None)      # float [nq] or None: one more term exp(sink) in every softmax denominator
     if not K.mfma_attention_supported(qkv.dtype, att.d, ctx.page_size):
         K.paged_attention_generic(
             out, qkv, q_row_stride, mem.pages["k"], mem.pages["v"], ctx.block_tables[mem.group], ctx.token_req,
-            ctx.positions, att.nq, att.nkv, att.d, att.scale, att.window or 0,
+            ctx.positions, att.nq, att.nkv, att.d, att.scale, att.window or 0, sinks=sinks,
         )
         return
     key = ("mfma_attention_plan", att.nq, att.nkv, att.d, bool(att.window))
@@ -160,8 +161,8 @@ def run(att, out, qkv, ctx, mem) -> None:
     if plan.n_prefill:
         K.attn_prefill_mfma(out, qkv, q_row_stride, mem.pages["k"], mem.pages["v"], tables, ctx.cu_seqlens,
                             ctx.context_lens, plan.prefill_work, plan.n_prefill, att.nq, att.nkv, att.d, att.scale,
-                            att.window or 0)
+                            att.window or 0, sinks=sinks)
     if plan.n_decode:
         K.attn_decode_mfma(out, qkv, q_row_stride, mem.pages["k"], mem.pages["v"], tables, ctx.cu_seqlens,
                            ctx.context_lens, plan.decode_work, plan.n_decode, att.nq, att.nkv, att.d, att.scale,
-                           att.window or 0, plan.num_splits, plan.scratch)
+                           att.window or 0, plan.num_splits, plan.scratch, sinks=sinks)

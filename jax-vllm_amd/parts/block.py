@@ -5,6 +5,11 @@
 The residual stream ``h`` is float.  Each sublayer's output is not added at once:
 it is handed on as ``delta`` and added inside the next norm's kernel (one pass over
 ``h`` instead of two), so a block takes and returns ``(h, delta)``.
+
+With ``residual_scale`` m every sublayer's output joins the stream times that constant,
+``h = h + m * mixer(norm_1(h))``: the output travels as a ``K.PendingNorm`` without a weight and
+the next norm's kernel multiplies in float while it adds.  ``has_feed_forward`` False: the
+first line only.
 """
 from __future__ import annotations
 
@@ -16,33 +21,44 @@ from .spec import PartSpec, build_part, is_replayable, register_part
 
 class PreNormBlock:
     def __init__(self, norm: PartSpec, mixer_norm_name: str = "input_layernorm",
-                 feed_forward_norm_name: str = "post_attention_layernorm"):
+                 feed_forward_norm_name: str = "post_attention_layernorm", residual_scale: float = 1.0,
+                 has_feed_forward: bool = True):
+        self.has_feed_forward = bool(has_feed_forward)
+        self.residual_scale = float(residual_scale)
         self.mixer_norm = build_part("norm", norm)
-        self.feed_forward_norm = build_part("norm", norm)
-        self.names = (mixer_norm_name, feed_forward_norm_name)
+        self.feed_forward_norm = build_part("norm", norm) if self.has_feed_forward else None
+        self.names = (mixer_norm_name, feed_forward_norm_name) if self.has_feed_forward else (mixer_norm_name,)
+        self.norms = (self.mixer_norm, self.feed_forward_norm) if self.has_feed_forward else (self.mixer_norm,)
 
     @property
     def replayable(self) -> bool:
-        return is_replayable(self.mixer_norm) and is_replayable(self.feed_forward_norm)
+        return all(is_replayable(n) for n in self.norms)
 
     def tensors(self) -> dict:
         out = {}
-        for name, part in zip(self.names, (self.mixer_norm, self.feed_forward_norm)):
+        for name, part in zip(self.names, self.norms):
             for k, v in part.tensors().items():
                 out[f"{name}.{k}"] = v
         return out
 
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
-        for name, part in zip(self.names, (self.mixer_norm, self.feed_forward_norm)):
+        for name, part in zip(self.names, self.norms):
             part.bind({k[len(name) + 1:]: v for k, v in tensors.items() if k.startswith(name + ".")}, dtype)
+
+    def _share(self, out):
+        """What a sublayer returned, as the next norm takes it."""
+        if self.residual_scale != 1.0:
+            return K.pending_scale(out, self.residual_scale)
+        return out.settled() if isinstance(out, K.BiasedOutput) else out
 
     def forward(self, h, delta, mixer, feed_forward, ctx, mem):
         n = h.shape[0]
         x = _add_norm(self.mixer_norm, h, delta, mixer, n)
-        a = mixer.forward(x, ctx, mem)
+        a = self._share(mixer.forward(x, ctx, mem))
+        if not self.has_feed_forward:
+            return a
         y = _add_norm(self.feed_forward_norm, h, a, feed_forward, n)
-        f = feed_forward.forward(y, ctx)
-        return f.settled() if isinstance(f, K.BiasedOutput) else f
+        return self._share(feed_forward.forward(y, ctx))
 
 
 def _add_norm(norm, h, delta, reader, n_rows: int):
@@ -51,7 +67,8 @@ def _add_norm(norm, h, delta, reader, n_rows: int):
     ``unscaled_ok``), a reader part answers ``takes_unscaled_rows(rows)``.  Parts that declare
     neither see the plain interface."""
     ask = getattr(reader, "takes_unscaled_rows", None)
-    if getattr(norm, "may_leave_scale", False) and ask is not None and ask(n_rows):
+    if (getattr(norm, "may_leave_scale", False) and ask is not None and not isinstance(delta, K.PendingNorm)
+            and ask(n_rows)):
         return norm.add_norm(h, delta, unscaled_ok=True)
     return norm.add_norm(h, delta)
 
@@ -139,7 +156,8 @@ class OutputNormBlock:
         if not isinstance(delta, K.PendingNorm):
             raise TypeError("this arrangement follows layers that hand on a sublayer's output with its norm")
         out = torch.empty(h.shape, dtype=self.dtype, device=h.device)
-        K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, None, out, bias=delta.bias)
+        K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, None, out, bias=delta.bias,
+                               plain_scale=delta.scale)
         return out
 
     def forward(self, h, delta, mixer, feed_forward, ctx, mem):

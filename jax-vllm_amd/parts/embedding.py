@@ -12,8 +12,10 @@ from .spec import TensorSpec, register_part
 class TokenEmbedding:
     replayable = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0):
+        """``scale``: a constant on every row, multiplied in float."""
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.scale = float(scale)
         self.weight = None
 
     def tensors(self) -> dict:
@@ -27,7 +29,12 @@ class TokenEmbedding:
         gives a row of NaN).  ``ctx`` is the step's ``StepContext`` (positions, token -> request, ...);
         this embedding needs none of it."""
         h = torch.empty((ids.numel(), self.hidden_size), dtype=torch.float32, device=ids.device)
-        K.embedding(h, self.weight, ids)
+        if self.scale != 1.0:
+            if ctx is None or ctx.prev_tokens is None:
+                raise ValueError("a scaled embedding runs through the pair kernel, which reads StepContext.prev_tokens")
+            K.embedding_pair(h, self.weight, None, ids, ctx.prev_tokens, 1, 0, 0, scale=self.scale)
+        else:
+            K.embedding(h, self.weight, ids)
         return h
 
 
@@ -36,11 +43,12 @@ class TokenPairEmbedding(TokenEmbedding):
     row ``(previous * mul_prev + token * mul_cur) mod buckets``; a sequence's first token takes the table's
     spare last row (number ``buckets``).  The previous token of every token of the step comes with the step's
     context (``StepContext.prev_tokens``, -1 for a first token): for the first token of a portion it is the last
-    token the cache manager holds for the request.  The sum is float."""
+    token the cache manager holds for the request.  ``scale``: a constant on the token's own row (not on the pair's).
+    The sum is float."""
 
     def __init__(self, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int, mul_cur: int,
-                 pair_name: str = "pair.weight"):
-        super().__init__(vocab_size, hidden_size)
+                 pair_name: str = "pair.weight", scale: float = 1.0):
+        super().__init__(vocab_size, hidden_size, scale)
         self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
         if self.buckets < 1 or self.mul_prev < 0 or self.mul_cur < 0:
             raise ValueError("buckets must be positive and the multipliers non-negative")
@@ -60,7 +68,8 @@ class TokenPairEmbedding(TokenEmbedding):
         if ctx is None or ctx.prev_tokens is None:
             raise ValueError("this embedding needs every token's previous token (StepContext.prev_tokens)")
         h = torch.empty((ids.numel(), self.hidden_size), dtype=torch.float32, device=ids.device)
-        K.embedding_pair(h, self.weight, self.pair, ids, ctx.prev_tokens, self.buckets, self.mul_prev, self.mul_cur)
+        K.embedding_pair(h, self.weight, self.pair, ids, ctx.prev_tokens, self.buckets, self.mul_prev, self.mul_cur,
+                         scale=self.scale)
         return h
 
 

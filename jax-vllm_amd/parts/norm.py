@@ -52,7 +52,7 @@ class RMSNorm:
             n_out = h.shape[0] if rows is None else rows.numel()
             out = torch.empty((n_out, self.size), dtype=self.dtype, device=h.device)
             K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, self.weight, out, rows, out_eps=self.eps,
-                                   bias=delta.bias)
+                                   bias=delta.bias, plain_scale=delta.scale)
             return out
         if (unscaled_ok and rows is None and delta is not None and delta.dim() == 3
                 and K.unscaled_rows_possible(self.dtype, h.shape[0], self.size)):

@@ -14,6 +14,9 @@ and differ in what q, k, v, the decay g and the write strength w are made of:
                    from a projection of its own, w = sigmoid(another projection); delta = 1; every head's o normed with a
                    weight shared by the heads, times silu(gate).
 
+A fourth mixer, ``time_mix`` (below), has a recurrence of its own, ``K.wkv_steps``: a decay per key channel instead of
+one per head, the output read from the state BEFORE the token's update, and a bonus on the token's own key.
+
 Everything that enters the recurrence is float (the products and the convolutions' results are in the activation
 type).  The state, and the last taps - 1 inputs of every convolution, live in the request's state slot between steps.
 """
@@ -199,6 +202,75 @@ class GatedDeltaMixer:
         return K.linear(y, self.w_o, partial_ok=True)
 
 
+class TimeMix:
+    """Time mixing with token shift, a data-dependent decay per key channel and a bonus for the current token.  With h_t
+    the mixer's input and h_(t-1) the row before it in the request (zeros before the first token), each of r, k, v, g, w
+    reads a blend of its own, b_s = h_t + (h_(t-1) - h_t) * mu_s:
+
+        r, k, v = W_r b_r, W_k b_k, W_v b_v  [heads, dim];   gate = silu(W_g b_g)
+        decay   = exp(-exp(W_w2 tanh(W_w1 b_w) + w0))         per head and key channel, float
+        o_t     = S^T r_t + (sum_d r_t[d] u[d] k_t[d]) v_t;    S <- diag(decay_t) S + k_t v_t^T      per head, S [dim, dim] float
+        out     = W_o ( concat_h( o_t / rms(o_t) ) * norm * gate )
+
+    The state S and the last input row h live in the request's state slot between steps (``S`` and ``shift``)."""
+
+    replayable = True     # slots, request borders and tokens come from the device; the kernel choice does not depend on values
+
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, norm_eps: float, decay_rank: Optional[int] = None):
+        """``decay_rank`` None: the inner size of the decay's two products is whatever the checkpoint's tensors have."""
+        self.hidden_size, self.heads, self.dim = int(hidden_size), int(num_heads), int(head_dim)
+        self.decay_rank, self.eps = int(decay_rank) if decay_rank else None, float(norm_eps)
+        if self.dim > K.WKV_MAX_DIM:
+            raise ValueError(f"the recurrence keeps heads of at most {K.WKV_MAX_DIM} channels, not {self.dim}")
+        self.inner = self.heads * self.dim
+
+    def tensors(self) -> dict:
+        hid, inner = self.hidden_size, self.inner
+        t = {f"mu.{s}": TensorSpec((hid,), role="vector", init="small") for s in self.MIXES}
+        t.update({
+            "r_proj.weight": TensorSpec((inner, hid)),
+            "k_proj.weight": TensorSpec((inner, hid)),
+            "v_proj.weight": TensorSpec((inner, hid)),
+            "gate.weight": TensorSpec((inner, hid)),
+            "decay_down.weight": TensorSpec((self.decay_rank, hid)),
+            "decay_up.weight": TensorSpec((inner, self.decay_rank)),
+            "decay_base": TensorSpec((inner,), role="vector", init="small"),
+            "bonus": TensorSpec((self.heads, self.dim), role="vector", init="small"),
+            "norm.weight": TensorSpec((inner,), role="vector", init="norm"),
+            "o_proj.weight": TensorSpec((hid, inner)),
+        })
+        return t
+
+    def cache_spec(self):
+        return None
+
+    def state_spec(self):
+        return (StateSpec((self.heads, self.dim, self.dim), "float32", "S"),
+                StateSpec((self.hidden_size,), "float32", "shift"))
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        self.dtype = dtype
+        self.mu = torch.stack([tensors[f"mu.{s}"] for s in self.MIXES]).contiguous()
+        self.w_r, self.w_k, self.w_v, self.w_g = (tensors[k + ".weight"] for k in ("r_proj", "k_proj", "v_proj", "gate"))
+        self.w_decay_down, self.w_decay_up = tensors["decay_down.weight"], tensors["decay_up.weight"]
+        self.decay_base = tensors["decay_base"].contiguous()
+        self.bonus = tensors["bonus"].reshape(-1).contiguous()
+        self.norm_weight, self.w_o = tensors["norm.weight"], tensors["o_proj.weight"]
+
+    def forward(self, x, ctx: StepContext, mem: LayerMemory):
+        H, d = self.heads, self.dim
+        b = K.token_shift_mix(x, self.mu, mem.states["shift"], ctx.slot_ids, ctx.cu_seqlens, ctx.token_req)
+        r, k, v, gate = (K.linear(b[i], w) for i, w in enumerate((self.w_r, self.w_k, self.w_v, self.w_g)))
+        low = K.linear(b[4], self.w_decay_down)
+        K.bias_act(low, None, "tanh")
+        rate = K.linear(low, self.w_decay_up)
+        o = K.wkv_steps(r, k, v, rate, self.decay_base, self.bonus, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, d, d)
+        y = K.group_gated_norm(o, gate, self.norm_weight, d, self.eps, "silu")
+        return K.linear(y, self.w_o, partial_ok=True)
+
+
 class ParallelMixer:
     """Two mixers side by side on the same input: ``left_scale * left(x) + right_scale * right(x)``.  Either may keep
     pages, either may keep state (their state tensors are declared under ``left.`` and ``right.``); their results
@@ -241,4 +313,5 @@ class ParallelMixer:
 register_part("mixer", "retention", Retention)
 register_part("mixer", "state_space", StateSpaceMixer)
 register_part("mixer", "gated_delta", GatedDeltaMixer)
+register_part("mixer", "time_mix", TimeMix)
 register_part("mixer", "parallel", ParallelMixer)

@@ -24,6 +24,8 @@ class TensorSpec:
            "vector"  – a small floating tensor always held in float32 (norm weights and the like:
                         a checkpoint's 32-bit values stay 32-bit, 16-bit values widen exactly);
            "table"   – an integer table, held as int32.
+    A ``None`` in ``shape`` is a size that only the checkpoint gives (the part reads it off the tensor it is bound
+    to); random weights need every size.
     init:  how the random-weights mode fills it: "normal" N(0, std), "norm" 1 + N(0, norm_std), "small"
            N(0, norm_std), "log_rate" -3 + N(0, 1), "zeros", or "index" (0, 1, 2, ... for integer tables).
     """

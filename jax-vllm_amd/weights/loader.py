@@ -73,7 +73,7 @@ def check_against_specs(where, specs: dict, ignored: set, available: dict, stric
         if name not in available:
             continue
         dtype, shape = available[name]
-        if tuple(shape) != tuple(ts.shape):
+        if len(shape) != len(ts.shape) or any(w is not None and g != w for g, w in zip(shape, ts.shape)):
             wrong_shape.append((name, tuple(shape), tuple(ts.shape)))
         is_float = dtype.is_floating_point
         if (ts.role == "table") == is_float:

@@ -26,6 +26,9 @@ def _tensor_seed(seed: int, name: str) -> int:
 
 
 def _draw(ts, seed: int, name: str, std: float, norm_std: float, device="cpu") -> torch.Tensor:
+    if any(d is None for d in ts.shape):
+        raise ValueError(f"random weights need every size: the configuration leaves a size of {name} {list(ts.shape)} to a "
+                         "checkpoint (give the mixer's optional size key)")
     g = torch.Generator(device=device).manual_seed(_tensor_seed(seed, name))
     if ts.init == "normal":
         return torch.randn(ts.shape, generator=g, dtype=torch.float32, device=device) * std
@@ -54,6 +57,8 @@ def write_random_model(folder, config: Mapping, seed: int, std: float = 0.02, no
     records = []
     for name, ts in sorted(model.tensor_specs().items()):
         dt = torch.int32 if ts.role == "table" else store
+        if any(d is None for d in ts.shape):
+            _draw(ts, seed, name, std, norm_std)      # raises: which size the configuration has to give
         records.append((name, tuple(ts.shape), dt,
                         lambda ts=ts, name=name, dt=dt: _draw(ts, seed, name, std, norm_std).to(dt)))
     (folder / "config.json").write_text(json.dumps(dict(raw), indent=2))
