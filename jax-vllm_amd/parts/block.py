@@ -47,7 +47,7 @@ class PreNormBlock:
 
     def _share(self, out):
         """What a sublayer returned, as the next norm takes it."""
-        if self.residual_scale != 1.0:
+        if self.residual_scale != 1.0 or isinstance(out, tuple):       # a pair (rows, float shares) is added there too
             return K.pending_scale(out, self.residual_scale)
         return out.settled() if isinstance(out, K.BiasedOutput) else out
 

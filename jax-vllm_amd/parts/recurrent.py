@@ -228,7 +228,7 @@ class TimeMix:
 
     def tensors(self) -> dict:
         hid, inner = self.hidden_size, self.inner
-        t = {f"mu.{s}": TensorSpec((hid,), role="vector", init="small") for s in self.MIXES}
+        t = {f"mu.{s}": TensorSpec((hid,), role="vector", init="fraction") for s in self.MIXES}
         t.update({
             "r_proj.weight": TensorSpec((inner, hid)),
             "k_proj.weight": TensorSpec((inner, hid)),
@@ -236,8 +236,8 @@ class TimeMix:
             "gate.weight": TensorSpec((inner, hid)),
             "decay_down.weight": TensorSpec((self.decay_rank, hid)),
             "decay_up.weight": TensorSpec((inner, self.decay_rank)),
-            "decay_base": TensorSpec((inner,), role="vector", init="small"),
-            "bonus": TensorSpec((self.heads, self.dim), role="vector", init="small"),
+            "decay_base": TensorSpec((inner,), role="vector", init="log_rate"),
+            "bonus": TensorSpec((self.heads, self.dim), role="vector", init="norm"),
             "norm.weight": TensorSpec((inner,), role="vector", init="norm"),
             "o_proj.weight": TensorSpec((hid, inner)),
         })

@@ -27,7 +27,7 @@ class TensorSpec:
     A ``None`` in ``shape`` is a size that only the checkpoint gives (the part reads it off the tensor it is bound
     to); random weights need every size.
     init:  how the random-weights mode fills it: "normal" N(0, std), "norm" 1 + N(0, norm_std), "small"
-           N(0, norm_std), "log_rate" -3 + N(0, 1), "zeros", or "index" (0, 1, 2, ... for integer tables).
+           N(0, norm_std), "log_rate" -3 + N(0, 1), "fraction" U(0, 1), "zeros", or "index" (0, 1, 2, ... for integer tables).
     """
 
     shape: tuple

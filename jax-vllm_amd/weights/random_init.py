@@ -38,6 +38,8 @@ def _draw(ts, seed: int, name: str, std: float, norm_std: float, device="cpu") -
         return torch.randn(ts.shape, generator=g, dtype=torch.float32, device=device) * norm_std
     if ts.init == "log_rate":     # the logarithm of a decay rate: rates around e^-3, a factor e either way
         return torch.randn(ts.shape, generator=g, dtype=torch.float32, device=device) - 3.0
+    if ts.init == "fraction":     # a blend weight between 0 and 1
+        return torch.rand(ts.shape, generator=g, dtype=torch.float32, device=device)
     if ts.init == "zeros":
         return torch.zeros(ts.shape, dtype=torch.float32, device=device)
     if ts.init == "index":

@@ -53,10 +53,10 @@ def test_config_validation():
 
 def test_registry_errors_match_reference_wording():
     """jllm/model/weights.py:59-65 and :161-170."""
-    assert supported_architectures() == ["Bozisun", "Dumazen", "Lomozen", "Qwen3ForCausalLM"]
+    assert supported_architectures() == ["Bozisun", "Dumazen", "Lomozen", "Qwen3ForCausalLM", "Zeripel"]
     with pytest.raises(ConfigError, match="no 'architectures' field"):
         resolve({k: v for k, v in TINY_A["config"].items() if k != "architectures"})
-    with pytest.raises(ConfigError, match="unsupported architecture: 'Qwen2ForCausalLM'.*Supported: Bozisun, Dumazen, Lomozen, Qwen3ForCausalLM"):
+    with pytest.raises(ConfigError, match="unsupported architecture: 'Qwen2ForCausalLM'.*Supported: Bozisun, Dumazen, Lomozen, Qwen3ForCausalLM, Zeripel"):
         resolve(dict(TINY_A["config"], architectures=["Qwen2ForCausalLM"]))
 
 
