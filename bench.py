@@ -86,6 +86,30 @@ def bozisun_shape(width, layers, heads, ff, experts, top, expert_ff, loop, vocab
             "layers": [dict(att, mlp=mlps[i % 2]) for i in range(layers)]}
 
 
+def zeripel_shape(width, layers, heads, ff, experts, top, expert_ff, shared_ff, vocab=32000):
+    """Layers in the order time mixing (heads of 64, as published models of that kind have), latent attention (a cached
+    vector of 224 + 32 elements), grouped-query attention with heads of 128 whose values are its keys, and latent
+    attention on the cache of the one two layers before; the time-mixing layers have a gated feed-forward, the others
+    routed experts with a shared expert (top * expert + shared = ff); a row per token pair."""
+    wkv = {"type": "wkv", "mixer": {"heads": width // 64, "dim": 64, "decay_rank": 64}}
+    latent = {"heads": heads, "dim": 64, "rot_dim": 32, "vdim": 64, "kv_rank": 224, "scale": 96 ** -0.5,
+              "rot": {"base": 500000.0, "dims": 32}}
+    att = {"type": "attention", "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128,
+                                          "scale": 128 ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}}}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top, "scale": 1.5}, "expert": {"ff": expert_ff},
+           "shared": {"ff": shared_ff}}
+    out = []
+    for i in range(layers):
+        if i % 4 == 0:
+            out.append(dict(wkv, mlp={"kind": "dense", "ff": ff}))
+        elif i % 4 == 2:
+            out.append(dict(att, mlp=moe))
+        else:
+            out.append({"type": "latent_attention", "mixer": dict(latent, **({"kv_from": i - 2} if i % 4 == 3 else {})), "mlp": moe})
+    return {"architecture": "Zeripel", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 100003, "mul_prev": 1000003, "mul_cur": 7919}}, "layers": out}
+
+
 # --only design: Lomozen beside the dense model of the same width, depth, vocabulary and feed-forward
 # parameters per token (top * expert + shared = intermediate)
 DESIGN_SHAPES = {
@@ -107,6 +131,12 @@ DUMAZEN_SHAPES = {
 BOZISUN_SHAPES = {
     "2k": (bozisun_shape(2048, 6, 16, 3072, 32, 4, 768, (2, 4, 2)),) + DESIGN_SHAPES["2k"],
     "4k": (bozisun_shape(4096, 6, 32, 8192, 64, 8, 1024, (2, 4, 2)),) + DESIGN_SHAPES["4k"],
+}
+# --only design --design zeripel: Zeripel beside Lomozen (the closest kin: latent attention, a linear recurrence with a state
+# per request, routed experts with a shared one) and the dense model, all of one width, depth and vocabulary
+ZERIPEL_SHAPES = {
+    "2k": (zeripel_shape(2048, 8, 16, 3072, 32, 4, 512, 1024),) + DESIGN_SHAPES["2k"],
+    "4k": (zeripel_shape(4096, 8, 32, 8192, 64, 6, 1024, 2048),) + DESIGN_SHAPES["4k"],
 }
 PROMPT_LEN = 1024
 MAX_CONTEXT = 8192
@@ -234,6 +264,7 @@ def measure_design(args, rng):
     out = {"shape": args.design_shape, "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_prompt_len": PROMPT_LEN}
     models = (zip(("dumazen", "lomozen", "dense"), DUMAZEN_SHAPES[args.design_shape]) if args.design == "dumazen"
               else zip(("bozisun", "lomozen", "dense"), BOZISUN_SHAPES[args.design_shape]) if args.design == "bozisun"
+              else zip(("zeripel", "lomozen", "dense"), ZERIPEL_SHAPES[args.design_shape]) if args.design == "zeripel"
               else zip(("lomozen", "dense"), DESIGN_SHAPES[args.design_shape]))
     out["design"] = args.design
     for name, cfg in models:
@@ -403,7 +434,7 @@ def main():
     ap.add_argument("--no-kernel-share", action="store_true", help="leave out the per-kernel time shares")
     ap.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k",
                     help="with --only design: the width of both models (2,048 or 4,096), 8 layers each")
-    ap.add_argument("--design", choices=["lomozen", "dumazen", "bozisun"], default="lomozen",
+    ap.add_argument("--design", choices=["lomozen", "dumazen", "bozisun", "zeripel"], default="lomozen",
                     help="with --only design: the architecture that is measured beside its kin of equal size")
     ap.add_argument("--design-models", default="", help="with --only design: only these of the models, with commas between them")
     ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt", "ttft", "calibrate", "design"], default=None,

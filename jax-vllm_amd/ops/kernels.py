@@ -1429,11 +1429,38 @@ def token_shift_mix(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, slot
 WKV_MAX_DIM = 8192      # 32 rows of a column in each of a block's 256 threads
 
 
-def wkv_steps(r, k, v, rate, w0, bonus, state, slot_ids, cu_seqlens, heads: int, dim: int, vdim: int) -> torch.Tensor:
+WKV_CHUNK_MIN_TOKENS = 8      # from this many tokens of a request on, the kernels by chunks
+WKV_CHUNK_MAX_DIM = 128       # key channels of a head whose chunk fits a block's LDS
+WKV_CHUNK_TOKENS = 32
+
+
+def wkv_chunk_plan(ctx, dim: int):
+    """The chunk plan of a step for ``wkv_steps`` (work int32 [chunks, 2] = (request, first token row), first chunk of
+    every request int32 [requests + 1], chunks), or None where the step runs token by token: a recorded step, a step of
+    short portions only, heads wider than the kernels by chunks take.  One plan serves every such layer of the step."""
+    if ctx.captured or ctx.max_q_len < WKV_CHUNK_MIN_TOKENS or dim > WKV_CHUNK_MAX_DIM:
+        return None
+    plan = ctx.plans.get("wkv_chunks")
+    if plan is None:
+        _need(int(library.core().jv_wkv_chunk_tokens()) == WKV_CHUNK_TOKENS, "the library's chunks have another size")
+        work, first, at = [], [0], 0
+        for r, n in enumerate(ctx.q_lens_host):
+            work += [(r, at + b) for b in range(0, n, WKV_CHUNK_TOKENS)]
+            first.append(len(work))
+            at += n
+        flat = torch.tensor([x for w in work for x in w] + first, dtype=torch.int32).pin_memory().to(ctx.positions.device, non_blocking=True)
+        plan = ctx.plans["wkv_chunks"] = (flat[:2 * len(work)], flat[2 * len(work):], len(work))
+    return plan
+
+
+def wkv_steps(r, k, v, rate, w0, bonus, state, slot_ids, cu_seqlens, heads: int, dim: int, vdim: int,
+              chunk_plan=None) -> torch.Tensor:
     """The recurrence with a decay per key channel and a bonus for the current token, per head with S the request's
     float state [dim, vdim]:  w = exp(-exp(rate + w0));  o = S^T r + (sum_d r[d] bonus[d] k[d]) v;  S <- diag(w) S + k v^T.
     r, k, rate [n, heads * dim] and v [n, heads * vdim] are views (unit column stride) of the activation type; w0 and
-    bonus float32 [heads * dim]; ``state`` float32 [slots + 1, heads, dim, vdim].  Returns float32 [n, heads * vdim]."""
+    bonus float32 [heads * dim]; ``state`` float32 [slots + 1, heads, dim, vdim].  Returns float32 [n, heads * vdim].
+    With ``chunk_plan`` (``wkv_chunk_plan``) the chunks of every request run side by side and only the states between
+    them are walked in order; the results differ from the token-by-token kernel's by rounding."""
     _dev(w0, bonus, state, slot_ids, cu_seqlens)
     n = r.shape[0]
     for name, t, width in (("r", r, heads * dim), ("k", k, heads * dim), ("rate", rate, heads * dim), ("v", v, heads * vdim)):
@@ -1446,6 +1473,22 @@ def wkv_steps(r, k, v, rate, w0, bonus, state, slot_ids, cu_seqlens, heads: int,
     _i32(slot_ids, "slot_ids")
     _i32(cu_seqlens, "cu_seqlens", slot_ids.numel() + 1)
     out = torch.empty((n, heads * vdim), dtype=torch.float32, device=r.device)
+    if chunk_plan is not None:
+        work, req_chunks, chunks = chunk_plan
+        _need(dim <= WKV_CHUNK_MAX_DIM, "heads too wide for the kernels by chunks")
+        _i32(work, "work", 2 * chunks)
+        _i32(req_chunks, "req_chunks", slot_ids.numel() + 1)
+        floats = torch.empty(chunks * heads * dim * vdim + n * heads * dim + chunks * heads * dim, dtype=torch.float32,
+                             device=r.device)
+        scratch = floats[:chunks * heads * dim * vdim]
+        rq = floats[scratch.numel():scratch.numel() + n * heads * dim]
+        dtot = floats[scratch.numel() + rq.numel():]
+        fn = getattr(library.core(), f"jv_wkv_chunks_{_suffix(r.dtype)}")
+        _check(fn(_ptr(out), _ptr(r), c_longlong(r.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
+                  _ptr(rate), c_longlong(rate.stride(0)), _ptr(w0), _ptr(bonus), _ptr(state), _ptr(slot_ids), _ptr(cu_seqlens),
+                  c_int(slot_ids.numel()), c_int(heads), c_int(dim), c_int(vdim), c_int(chunks), _ptr(work), _ptr(req_chunks),
+                  _ptr(scratch), _ptr(rq), _ptr(dtot), _stream()), "wkv_chunks")
+        return out
     fn = getattr(library.core(), f"jv_wkv_steps_{_suffix(r.dtype)}")
     _check(fn(_ptr(out), _ptr(r), c_longlong(r.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
               _ptr(rate), c_longlong(rate.stride(0)), _ptr(w0), _ptr(bonus), _ptr(state), _ptr(slot_ids), _ptr(cu_seqlens),

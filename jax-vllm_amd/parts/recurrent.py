@@ -266,7 +266,8 @@ class TimeMix:
         low = K.linear(b[4], self.w_decay_down)
         K.bias_act(low, None, "tanh")
         rate = K.linear(low, self.w_decay_up)
-        o = K.wkv_steps(r, k, v, rate, self.decay_base, self.bonus, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, d, d)
+        o = K.wkv_steps(r, k, v, rate, self.decay_base, self.bonus, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, d, d,
+                        chunk_plan=K.wkv_chunk_plan(ctx, d))
         y = K.group_gated_norm(o, gate, self.norm_weight, d, self.eps, "silu")
         return K.linear(y, self.w_o, partial_ok=True)
 

@@ -518,21 +518,26 @@ def test_kernel_blends_with_the_row_before(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("shape", [(3, 8, 8), (1, 80, 80), (2, 128, 128), (5, 6, 6)])
-def test_kernel_recurrence_with_a_decay_per_channel_and_a_bonus(dtype, shape):
-    """Two requests (7 and 30 rows) that continue states of their own against the recurrence written out token by
-    token; the outputs and the states that the step leaves."""
+@pytest.mark.parametrize("chunks", [False, True], ids=["steps", "chunks"])
+@pytest.mark.parametrize("shape", [(3, 8, 8), (1, 80, 80), (2, 128, 128), (5, 6, 6), (2, 64, 72)])
+def test_kernel_recurrence_with_a_decay_per_channel_and_a_bonus(dtype, chunks, shape):
+    """Three requests (7, 1 and 100 rows: chunks that are full, short and single) that continue states of their own
+    against the recurrence written out token by token; the outputs and the states that the step leaves.  Some decays
+    are next to nothing (rates far above zero), some next to one."""
+    from types import SimpleNamespace
+
     from jax_vllm_amd.ops import kernels as K
 
     H, d, dv = shape
     g = torch.Generator().manual_seed(2)
-    lens, slots = [7, 30], [1, 0]
+    lens, slots = [7, 1, 100], [1, 3, 0]
     n = sum(lens)
     r, k, v = (torch.randn(n, H * s, generator=g).to(dtype) for s in (d, d, dv))
     rate = (torch.randn(n, H * d, generator=g) * 0.5).to(dtype)
+    rate[40:44] = 6.0           # these tokens wipe the state: log decays of -e^4 and below
     w0 = torch.randn(H * d, generator=g) - 2.0
     bonus = torch.randn(H * d, generator=g)
-    state = torch.randn(3, H, d, dv, generator=g)
+    state = torch.randn(5, H, d, dv, generator=g)
     want, want_state = torch.empty(n, H * dv, dtype=torch.float64), state.double().clone()
     cu = np.cumsum([0] + lens)
     for q, s in enumerate(slots):
@@ -545,12 +550,18 @@ def test_kernel_recurrence_with_a_decay_per_channel_and_a_bonus(dtype, shape):
             S = wt.unsqueeze(2) * S + kv
         want_state[s] = S
     st = _dev(state.clone())
+    plan = None
+    if chunks:
+        ctx = SimpleNamespace(captured=False, max_q_len=max(lens), plans={}, q_lens_host=lens, positions=st)
+        plan = K.wkv_chunk_plan(ctx, d)
+        assert plan is not None and plan[2] == 1 + 1 + 4
     got = K.wkv_steps(_dev(r), _dev(k), _dev(v), _dev(rate), _dev(w0), _dev(bonus), st,
-                      _dev(torch.tensor(slots, dtype=torch.int32)), _dev(torch.tensor(cu, dtype=torch.int32)), H, d, dv)
+                      _dev(torch.tensor(slots, dtype=torch.int32)), _dev(torch.tensor(cu, dtype=torch.int32)), H, d, dv,
+                      chunk_plan=plan)
     scale = float(want.abs().max())
     assert float((got.double().cpu() - want).abs().max()) <= 2e-5 * scale
     assert float((st.double().cpu() - want_state).abs().max()) <= 2e-5 * float(want_state.abs().max())
-    assert torch.equal(st[2].cpu(), state[2])
+    assert torch.equal(st[2].cpu(), state[2]) and torch.equal(st[4].cpu(), state[4])
 
 
 @pytest.mark.parametrize("n", [5, 40, 300])
