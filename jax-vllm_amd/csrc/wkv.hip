@@ -45,6 +45,44 @@ token_shift_mix_kernel(T* __restrict__ out, const T* __restrict__ x, const float
     out[((long long)s * n + t) * hidden + c] = from_f32<T>(fmaf(d, mu[(long long)s * hidden + c], cur));
 }
 
+// The same with 16 bytes a lane, where the width and the addresses allow it.
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_mix_vec_kernel(T* __restrict__ out, const T* __restrict__ x, const float* __restrict__ mu, int n_mix,
+                           float* __restrict__ state, const int* __restrict__ slot_ids,
+                           const int* __restrict__ cu_seqlens, const int* __restrict__ token_req, long long n,
+                           int hidden) {
+  constexpr int V = 16 / (int)sizeof(T);
+  typedef T tv __attribute__((ext_vector_type(V)));
+  const long long t = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * V;
+  if (c >= hidden) return;
+  const int r = token_req[t];
+  const int t0 = cu_seqlens[r], t1 = cu_seqlens[r + 1];
+  const tv cv = *(const tv*)(x + t * hidden + c);
+  float cur[V], d[V];
+  if (t > t0) {
+    const tv bv = *(const tv*)(x + (t - 1) * hidden + c);
+#pragma unroll
+    for (int e = 0; e < V; ++e) { cur[e] = to_f32(cv[e]); d[e] = to_f32(bv[e]) - cur[e]; }
+  } else {
+    float* st = state + (long long)slot_ids[r] * hidden + c;
+    const tv lv = *(const tv*)(x + (long long)(t1 - 1) * hidden + c);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      cur[e] = to_f32(cv[e]);
+      d[e] = st[e] - cur[e];
+      st[e] = to_f32(lv[e]);
+    }
+  }
+  for (int s = 0; s < n_mix; ++s) {
+    tv ov;
+#pragma unroll
+    for (int e = 0; e < V; ++e) ov[e] = from_f32<T>(fmaf(d[e], mu[(long long)s * hidden + c + e], cur[e]));
+    *(tv*)(out + ((long long)s * n + t) * hidden + c) = ov;
+  }
+}
+
 // ---------------------------------------------------------------- the recurrence, token by token
 // grid (requests, heads, column slices); block 256 = parts x cols threads, cols a power of two.
 // r, k, rate: [n][heads][dim] with row strides ldr, ldk, ldw; v [n][heads][vdim] with row stride ldv; w0, u [heads][dim]
@@ -127,6 +165,10 @@ wkv_steps_kernel(float* __restrict__ out, const T* __restrict__ rr, long long ld
 #define WKV_CW 64          // columns of v a block takes at a time
 #define WKV_MIN_LOG 64.f
 
+// e^x for x in [-32 * WKV_MIN_LOG, 0] through the hardware's 2^x: the argument's rounding costs |x| e^x 2^-24 at most,
+// below a hundred-millionth absolutely, which is the float rounding of the sums these weights enter.
+__device__ __forceinline__ float wkv_exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 wkv_local_kernel(float* __restrict__ out, float* __restrict__ scratch, float* __restrict__ rq, float* __restrict__ dtot,
@@ -134,14 +176,16 @@ wkv_local_kernel(float* __restrict__ out, float* __restrict__ scratch, float* __
                  const T* __restrict__ vv, long long ldv, const T* __restrict__ rate, long long ldw,
                  const float* __restrict__ w0, const float* __restrict__ bonus, const int* __restrict__ work,
                  const int* __restrict__ cu_seqlens, int heads, int dim, int vdim) {
-  extern __shared__ float lds[];      // r [LC][dim + 1] | k [LC][dim + 1] | b [LC][dim + 1] | a [LC][LC + 1] | v [LC][CW]
+  extern __shared__ float lds[];      // r [LC][dim + 1] | k [LC][dim + 1] | b [LC][dim + 1] | a [LC][LC + 1] | v [LC][CW] | u [dim]
   const int ld = dim + 1;
   float* rs = lds;
   float* ks = rs + WKV_LC * ld;
   float* bs = ks + WKV_LC * ld;
   float* as = bs + WKV_LC * ld;
   float* vs = as + WKV_LC * (WKV_LC + 1);
+  float* us = vs + WKV_LC * WKV_CW;
   const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  for (int c = tid; c < dim; c += 256) us[c] = bonus[h * dim + c];
   const int req = work[2 * ch], b0 = work[2 * ch + 1];
   const int n = min(WKV_LC, cu_seqlens[req + 1] - b0);
   for (int i = tid; i < WKV_LC * dim; i += 256) {
@@ -164,9 +208,9 @@ wkv_local_kernel(float* __restrict__ out, float* __restrict__ scratch, float* __
       const float before = run;
       run += bs[t * ld + c];
       bs[t * ld + c] = run;
-      if (t < n) rq[(long long)(b0 + t) * heads * dim + h * dim + c] = rs[t * ld + c] * expf(before);
+      if (t < n) rq[(long long)(b0 + t) * heads * dim + h * dim + c] = rs[t * ld + c] * wkv_exp_neg(before);
     }
-    dtot[((long long)ch * heads + h) * dim + c] = expf(run);
+    dtot[((long long)ch * heads + h) * dim + c] = wkv_exp_neg(run);
   }
   __syncthreads();
   for (int e = tid; e < WKV_LC * WKV_LC; e += 256) {
@@ -174,16 +218,16 @@ wkv_local_kernel(float* __restrict__ out, float* __restrict__ scratch, float* __
     float a = 0.f;
     if (j < t) {
       for (int c = 0; c < dim; ++c)
-        a = fmaf(rs[t * ld + c] * ks[j * ld + c], expf(bs[(t - 1) * ld + c] - bs[j * ld + c]), a);
+        a = fmaf(rs[t * ld + c] * ks[j * ld + c], wkv_exp_neg(bs[(t - 1) * ld + c] - bs[j * ld + c]), a);
     } else if (j == t) {
-      for (int c = 0; c < dim; ++c) a = fmaf(rs[t * ld + c] * ks[t * ld + c], bonus[h * dim + c], a);
+      for (int c = 0; c < dim; ++c) a = fmaf(rs[t * ld + c] * ks[t * ld + c], us[c], a);
     }
     as[t * (WKV_LC + 1) + j] = a;
   }
   __syncthreads();
   for (int i = tid; i < WKV_LC * dim; i += 256) {
     const int t = i / dim, c = i - t * dim;
-    ks[t * ld + c] *= expf(bs[(WKV_LC - 1) * ld + c] - bs[t * ld + c]);
+    ks[t * ld + c] *= wkv_exp_neg(bs[(WKV_LC - 1) * ld + c] - bs[t * ld + c]);
   }
   const int col = tid & (WKV_CW - 1), tq = tid / WKV_CW;      // tq is the same for all lanes of a wave
   for (int c0 = 0; c0 < vdim; c0 += WKV_CW) {
@@ -293,6 +337,13 @@ extern "C" int jv_wkv_chunk_max_dim() { return 128; }
                                           long long n, int hidden, void* stream) {                              \
     if (n <= 0 || hidden <= 0 || n_mix <= 0) return 0;                                                          \
     if (n > 0x7fffffffll || (hidden + 255) / 256 > 65535) return (int)hipErrorInvalidValue;                     \
+    constexpr int V = 16 / (int)sizeof(T);                                                                      \
+    if (hidden % V == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)x % 16 == 0) {                                \
+      hipLaunchKernelGGL(token_shift_mix_vec_kernel<T>, dim3((unsigned)n, (hidden / V + 255) / 256), dim3(256), \
+                         0, (hipStream_t)stream, (T*)out, (const T*)x, mu, n_mix, state, slot_ids, cu_seqlens,  \
+                         token_req, n, hidden);                                                                 \
+      return JV_LAUNCH_CHECK();                                                                                 \
+    }                                                                                                           \
     hipLaunchKernelGGL(token_shift_mix_kernel<T>, dim3((unsigned)n, (hidden + 255) / 256), dim3(256), 0,        \
                        (hipStream_t)stream, (T*)out, (const T*)x, mu, n_mix, state, slot_ids, cu_seqlens,       \
                        token_req, n, hidden);                                                                   \
@@ -331,7 +382,7 @@ extern "C" int jv_wkv_chunk_max_dim() { return 128; }
       return (int)hipErrorInvalidValue;                                                                         \
     if (((long long)dim * vdim + 255) / 256 > 65535) return (int)hipErrorInvalidValue;                          \
     hipStream_t s = (hipStream_t)stream;                                                                        \
-    const size_t lds_local = (3 * WKV_LC * (dim + 1) + WKV_LC * (WKV_LC + 1) + WKV_LC * WKV_CW) * sizeof(float); \
+    const size_t lds_local = (3 * WKV_LC * (dim + 1) + WKV_LC * (WKV_LC + 1) + WKV_LC * WKV_CW + dim) * sizeof(float); \
     hipLaunchKernelGGL(wkv_local_kernel<T>, dim3(chunks, heads), dim3(256), lds_local, s, out, scratch, rq, dtot, \
                        (const T*)r, ldr, (const T*)k, ldk, (const T*)v, ldv, (const T*)rate, ldw, w0, bonus,    \
                        work, cu_seqlens, heads, dim, vdim);                                                     \

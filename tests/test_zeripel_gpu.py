@@ -488,13 +488,14 @@ def _dev(x, dtype=None):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-def test_kernel_blends_with_the_row_before(dtype):
+@pytest.mark.parametrize("hidden", [50, 64, 520])
+def test_kernel_blends_with_the_row_before(dtype, hidden):
     """Three requests of 5, 1 and 12 rows in slots 2, 0 and 3: the first row of each blends with its slot's state row,
     which then holds the request's last row; other slots stay as they were."""
     from jax_vllm_amd.ops import kernels as K
 
     g = torch.Generator().manual_seed(1)
-    hidden, lens, slots = 50, [5, 1, 12], [2, 0, 3]
+    lens, slots = [5, 1, 12], [2, 0, 3]
     n = sum(lens)
     x = torch.randn(n, hidden, generator=g).to(dtype)
     mu = torch.rand(5, hidden, generator=g)
