@@ -744,10 +744,11 @@ def test_kernel_gates_of_a_head_and_of_a_row(dtype):
     want = torch.einsum("thk,hnk->thn", x.double().view(n, H, Kd), w.double()) * torch.sigmoid(gates.double()[:, 1:1 + H]).unsqueeze(-1)
     tol = 1e-5 if dtype == torch.float32 else 3e-2
     assert torch.allclose(y.double().cpu().view(n, H, N), want, atol=tol, rtol=tol)
-    rows = torch.randn(n, 50, generator=g).to(dtype)
-    out = torch.empty(n, 50, dtype=torch.float32, device="cuda")
-    K.row_gate(out, _dev(rows), _dev(gates)[:, 2:3])
-    assert torch.allclose(out.cpu().double(), rows.double() * torch.sigmoid(gates.double()[:, 2:3]), atol=1e-6, rtol=1e-6)
+    for width in (50, 64):
+        rows = torch.randn(n, width, generator=g).to(dtype)
+        out = torch.empty(n, width, dtype=torch.float32, device="cuda")
+        K.row_gate(out, _dev(rows), _dev(gates)[:, 2:3])
+        assert torch.allclose(out.cpu().double(), rows.double() * torch.sigmoid(gates.double()[:, 2:3]), atol=1e-6, rtol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
